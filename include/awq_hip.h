@@ -1,0 +1,192 @@
+/*
+ * awq_hip.h -- C-ABI of libawq_hip.so: AWQ int4 group-128 weight-only batch-1
+ * decode on one AMD gfx950 GPU.
+ *
+ * The reference (llama_cu_awq) has no FFI or plugin interface: its host code
+ * launches kernels through a set of static launcher functions in one
+ * translation unit.  This header cuts the seam there.  Each entry point below
+ * names the reference launcher / call site it replaces (paths relative to the
+ * reference checkout) and keeps that launcher's argument meaning.
+ *
+ * Conventions (the reference's):
+ *   - every op is asynchronous on the context's single stream and never
+ *     synchronises; only awq_stream_sync() and the blocking copies wait;
+ *   - the caller owns every buffer; ops own nothing;
+ *   - the sequence position is passed as a DEVICE pointer and read inside the
+ *     kernels, so that a recorded launch sequence can be replayed;
+ *   - fp16 tensors are passed as uint16_t* (IEEE binary16 bit patterns);
+ *   - a packed matrix with reduction length K and N outputs is three arrays,
+ *     one row per output n:
+ *       weight[n*pwh + k/8]  uint32, element k in bits 4*(k%8), pwh = ceil(K/32)*4
+ *       zeros [n*pzh + g/8]  uint32, group g = k/128 in bits 4*(g%8), pzh = ceil(ceil(K/128)/8)
+ *       scales[n*sh  + g]    fp16,   sh = ceil(K/128)
+ *     (common.h:26-30, llama2_q4.cu:106-129, weight_packer.cpp:114-124).
+ *
+ * Every function returns AWQ_OK (0) or a negative status; it never exits the
+ * process.  Where the reference prints "Unsupported matmul size. Exiting" and
+ * exits (K or N not a multiple of 8), this library returns AWQ_ERR_SHAPE and
+ * launches nothing.  The library is thread-agnostic: a context may be used
+ * from any one thread at a time; there is no thread-local state.
+ */
+#ifndef AWQ_HIP_H
+#define AWQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AWQ_OK 0
+#define AWQ_ERR_ARG (-1)    /* null pointer / bad argument */
+#define AWQ_ERR_SHAPE (-2)  /* the reference's "Unsupported matmul size" guard, or a size a kernel cannot take */
+#define AWQ_ERR_HIP (-3)    /* a HIP runtime call failed; see awq_last_error() */
+#define AWQ_ERR_IO (-4)     /* model file missing / short / bad header */
+
+typedef struct awq_ctx awq_ctx;                 /* device ordinal + stream + library workspace */
+typedef struct awq_transformer awq_transformer; /* weights + run state of one model on one GPU */
+
+/* Text of the most recent error recorded by any call in this process. */
+const char* awq_last_error(void);
+
+/* ---- context: cudaSetDevice + cudaStreamCreate (llama2_q4.cu:685, 695) and the
+ *      global `streams[rank]` (llama2_q4.cu:338-345). */
+int awq_ctx_create(int device, awq_ctx** out);
+/* Same, but enqueue on a stream the caller owns (a hipStream_t), e.g. torch's current stream. */
+int awq_ctx_create_on_stream(int device, void* hip_stream, awq_ctx** out);
+int awq_ctx_destroy(awq_ctx* ctx);
+/* cudaStreamSynchronize (llama2_q4.cu:713, 737). */
+int awq_stream_sync(awq_ctx* ctx);
+/* Raw hipStream_t of the context. */
+void* awq_ctx_stream(awq_ctx* ctx);
+
+/* ---- memory: cudaMalloc / cudaFree / cudaMallocHost / cudaFreeHost / cudaMemcpyAsync /
+ *      cudaMemset (llama2_q4.cu:62-74, 93-104, 114-136, 249, 703). */
+int awq_malloc(awq_ctx* ctx, void** ptr, size_t bytes);
+int awq_free(awq_ctx* ctx, void* ptr);
+int awq_malloc_host(awq_ctx* ctx, void** ptr, size_t bytes); /* pinned, GPU-visible */
+int awq_free_host(awq_ctx* ctx, void* ptr);
+int awq_memcpy_h2d_async(awq_ctx* ctx, void* dst, const void* src, size_t bytes);
+int awq_memcpy_h2d(awq_ctx* ctx, void* dst, const void* src, size_t bytes); /* blocking */
+int awq_memcpy_d2h(awq_ctx* ctx, void* dst, const void* src, size_t bytes); /* blocking, ordered after the stream */
+int awq_memset_async(awq_ctx* ctx, void* dst, int value, size_t bytes);
+
+/* ---- timing on the context's stream (cudaEvent pair, llama2_q4.cu:545-550, 592-600). */
+int awq_event_create(awq_ctx* ctx, void** event);
+int awq_event_destroy(awq_ctx* ctx, void* event);
+int awq_event_record(awq_ctx* ctx, void* event);
+int awq_event_elapsed_ms(awq_ctx* ctx, void* start, void* stop, float* ms); /* waits for `stop` */
+
+typedef struct awq_qweight { /* QWeight, common.h:26-30 (device pointers) */
+    const uint32_t* weight;
+    const uint32_t* zeros;
+    const uint16_t* scales;
+} awq_qweight;
+
+/* ---- ops: the launchers of llama2_q4.cu:347-427 and sampler.h:77-84 ---- */
+
+/* copy_embedding_kernel launch, llama2_q4.cu:441: x[i] = table[tokens[*pos]*dim + i].
+ * `tokens` may be pinned host memory (as in the reference) or device memory. */
+int awq_embed(awq_ctx* ctx, uint16_t* x, const uint16_t* table, int dim, const int* tokens, const int* pos);
+
+/* rmsnorm(), llama2_q4.cu:347-350: o = half(x * (rsqrt(mean(x^2)+1e-5) * weight)); o may alias x. */
+int awq_rmsnorm(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const uint16_t* weight, int size);
+
+/* matmul(QWeight), llama2_q4.cu:367-376: out = half(W x), fp32 accumulation.
+ * accum != 0: out = half(W x + out/gpu_count) (fused residual; gpu_count is 1 on one GPU).
+ * loff != -1: the result row is written at out + loff + (*pos)*N (KV-cache row); pos may be NULL when loff == -1. */
+int awq_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* w, int K, int N,
+                    int accum, int gpu_count, int loff, const int* pos);
+
+/* qkv_matvec(), llama2_q4.cu:378-391: q = Wq x; key_cache[loff + pos*N ..] = Wk x; value_cache[...] = Wv x. */
+int awq_qkv_matvec(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
+                   const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw, int K, int N, int loff,
+                   const int* pos);
+
+/* ffn_matvec_silu(), llama2_q4.cu:393-404: out = half(silu(Wgate x) * (Wup x)), both products kept in fp32. */
+int awq_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w,
+                        const awq_qweight* up_w, int K, int N);
+
+/* RoPERotation(), llama2_q4.cu:406-408: rotate-half RoPE, pairs (i, i+head/2), in place on q (all heads)
+ * and on the K row at k + loff + (*pos)*num_kv_heads*head_size (first num_kv_heads heads). */
+int awq_rope(awq_ctx* ctx, uint16_t* q, uint16_t* k, int num_heads, int num_kv_heads, int head_size, const int* pos,
+             int loff, float rope_theta);
+
+/* MultiHeadAttention(), llama2_q4.cu:410-427.  key_cache / value_cache point at the layer's
+ * (seq_len, num_heads*head_size/kv_mul) block.  att is a scratch of num_heads*max_seq_len halves; on return it
+ * holds the fp16 scores with the reference's compact row stride (*pos + 1) (the reference overwrites them with
+ * the probabilities, which nothing reads afterwards).  max_seq_len only sizes the launch (any value > *pos);
+ * the live length is read from *pos on the device.  head_size must be 64, 128 or 256. */
+int awq_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const uint16_t* key_cache,
+                  const uint16_t* value_cache, uint16_t* att, int num_heads, int head_size, int kv_mul,
+                  int max_seq_len, const int* pos);
+
+/* matmul(half), llama2_q4.cu:357-365 as used for the classifier (:530): out[r] = half(sum_j w[r*n+j] x[j]),
+ * w row-major (d, n).  The batch/stride/alpha generality of the reference launcher is unused on its live path. */
+int awq_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d);
+
+/* sample() greedy branch, sampler.h:77-84 (argmax_kernel, gpu_kernels.h:456-501): index of the largest logit
+ * (lowest index on ties); p = *pos_dev + 1; if write_token, tokens[p] = argmax; *pos_host = *pos_dev = p.
+ * tokens and pos_host are pinned host memory in the reference; any GPU-visible memory works. */
+int awq_argmax_advance(awq_ctx* ctx, const uint16_t* logits, int size, int* tokens, volatile int* pos_host,
+                       int* pos_dev, int write_token);
+
+/* Dequantise a packed matrix to fp16, out[n*K + k] = half_rne((q - z) * scale): the arithmetic of
+ * gpu_kernels.h:204-205 materialised (no launcher in the reference; used by the prefill path and by tests). */
+int awq_dequant(awq_ctx* ctx, uint16_t* out, const awq_qweight* w, int K, int N);
+
+/* ---- model level: build_transformer / run_transformer / free_transformer ---- */
+
+typedef struct awq_config { /* Config, common.h:15-24 = the 32-byte file header */
+    int dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab_size, seq_len;
+    float rope_theta;
+} awq_config;
+
+typedef struct awq_run_state { /* RunState, common.h:62-78 (device pointers; shared_* are pinned host) */
+    uint16_t *x, *xb, *hb, *q, *att, *logits, *key_cache, *value_cache;
+    int* pos;                  /* device copy of the position */
+    volatile int* shared_pos;  /* SharedData.pos  (common.h:57-60) */
+    int* shared_tokens;        /* SharedData.tokens */
+} awq_run_state;
+
+typedef struct awq_layer_weights { /* PerLayerWeight, common.h:32-42 */
+    const uint16_t* rms_att_weight;
+    const uint16_t* rms_ffn_weight;
+    awq_qweight wq_q, wq_k, wq_v, wq_o, wq_gate, wq_up, wq_down;
+} awq_layer_weights;
+
+/* build_transformer(), llama2_q4.cu:625-659, single GPU: read the header and every tensor of a weight_packer
+ * .bin file (order llama2_q4.cu:220-246) to the GPU and allocate the run state (llama2_q4.cu:62-91). */
+int awq_transformer_load_file(awq_ctx* ctx, const char* checkpoint_path, awq_transformer** out);
+/* Same from a file image in host memory (synthetic models, tests). */
+int awq_transformer_load_image(awq_ctx* ctx, const void* image, size_t bytes, awq_transformer** out);
+/* free_transformer(), llama2_q4.cu:668-678. */
+int awq_transformer_free(awq_transformer* t);
+int awq_transformer_config(const awq_transformer* t, awq_config* out);
+int awq_transformer_state(const awq_transformer* t, awq_run_state* out);
+int awq_transformer_layer(const awq_transformer* t, int layer, awq_layer_weights* out);
+/* token_embedding_table, wcls, rms_final_weight (common.h:44-54). */
+int awq_transformer_globals(const awq_transformer* t, const uint16_t** embed, const uint16_t** wcls,
+                            const uint16_t** rms_final);
+
+/* Start a sequence (llama2_q4.cu:703-705): position 0, prompt copied into the shared token list. */
+int awq_transformer_reset(awq_transformer* t, const int* prompt_tokens, int num_prompt_tokens);
+/* Start at position `pos` with caller-provided KV-cache contents below it; `token` is consumed next. */
+int awq_transformer_set_pos(awq_transformer* t, int pos, int token);
+
+/* run_transformer(), llama2_q4.cu:541-601, with the greedy sampler: one token through the network
+ * (run_llama_network, llama2_q4.cu:430-538, gpu_count 1) followed by argmax-and-advance.
+ * gen_token: write the sampled token into the shared list (false while the prompt is being consumed).
+ * use_graph != 0 replays a recorded launch sequence keyed by sequence-length bin (the USE_CUDA_GRAPHS path,
+ * llama2_q4.cu:553-575); 0 launches eagerly.  mode selects the schedule: AWQ_SCHEDULE_REFERENCE issues the
+ * reference's op sequence one launcher at a time; AWQ_SCHEDULE_FUSED merges RMSNorm into the consuming
+ * matrix-vector kernels and RoPE into the QKV kernel (same rounding points). */
+#define AWQ_SCHEDULE_REFERENCE 0
+#define AWQ_SCHEDULE_FUSED 1
+int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AWQ_HIP_H */

@@ -1,0 +1,18 @@
+"""MI355X-native AWQ int4 group-128 batch-1 decode (host-side mirror of the C-ABI in include/awq_hip.h)."""
+from ._lib import AwqError, lib, lib_path  # noqa: F401
+from .ops import (  # noqa: F401
+    Context,
+    DeviceBuffer,
+    QWeight,
+    MultiHeadAttention,
+    RoPERotation,
+    argmax_advance,
+    copy_embedding,
+    dequant,
+    ffn_matvec_silu,
+    matmul,
+    matmul_q,
+    qkv_matvec,
+    rmsnorm,
+)
+from .model import Transformer, SCHEDULE_FUSED, SCHEDULE_REFERENCE  # noqa: F401

@@ -1,0 +1,137 @@
+// Shared host/device helpers of libawq_hip (gfx950, wave64 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/awq_hip.h"
+
+// ---------------------------------------------------------------- host side
+struct awq_ctx {
+    int device;
+    hipStream_t stream;
+    bool owns_stream;
+    // Library workspace for the split attention kernel: per-(head, split)
+    // partial outputs and one arrival counter per head (self-resetting).
+    float* attn_partial;
+    unsigned int* attn_counter;
+};
+
+constexpr int kAttnMaxHeads = 256;
+constexpr int kAttnMaxSplits = 16;
+constexpr int kAttnMaxHeadSize = 256;
+
+void awq_set_error(const char* fmt, ...);
+
+#define AWQ_HIP_TRY(expr)                                                                      \
+    do {                                                                                       \
+        hipError_t e_ = (expr);                                                                \
+        if (e_ != hipSuccess) {                                                                \
+            awq_set_error("%s:%d: %s failed: %s", __FILE__, __LINE__, #expr, hipGetErrorString(e_)); \
+            return AWQ_ERR_HIP;                                                                \
+        }                                                                                      \
+    } while (0)
+
+#define AWQ_REQUIRE(cond, code, msg)                   \
+    do {                                               \
+        if (!(cond)) {                                 \
+            awq_set_error("%s: %s", __func__, msg);    \
+            return code;                               \
+        }                                              \
+    } while (0)
+
+static inline int awq_bind(awq_ctx* ctx) {
+    if (!ctx) {
+        awq_set_error("null context");
+        return AWQ_ERR_ARG;
+    }
+    AWQ_HIP_TRY(hipSetDevice(ctx->device));
+    return AWQ_OK;
+}
+
+static inline int awq_check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        awq_set_error("launch of %s failed: %s", what, hipGetErrorString(e));
+        return AWQ_ERR_HIP;
+    }
+    return AWQ_OK;
+}
+
+static inline int div_up(int a, int b) { return (a + b - 1) / b; }
+// Derived strides of a packed matrix (see awq_hip.h).
+static inline int packed_weight_height(int K) { return div_up(K, 32) * 4; }
+static inline int scales_height(int K) { return div_up(K, 128); }
+static inline int packed_zeros_height(int K) { return div_up(scales_height(K), 8); }
+
+// Largest reduction length the matrix-vector kernels stage in LDS (fp16
+// activations, 2 bytes each, inside the 64 KB a workgroup may allocate).
+constexpr int kMaxStagedK = 28672;
+
+// ---------------------------------------------------------------- device side
+#ifdef __HIPCC__
+
+typedef _Float16 h16_t;
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ h16x2 as_h2(uint32_t u) { return __builtin_bit_cast(h16x2, u); }
+__device__ __forceinline__ uint32_t as_u32(h16x2 h) { return __builtin_bit_cast(uint32_t, h); }
+__device__ __forceinline__ float half_bits_to_float(uint16_t b) { return (float)__builtin_bit_cast(h16_t, b); }
+__device__ __forceinline__ uint16_t float_to_half_bits(float f) { return __builtin_bit_cast(uint16_t, (h16_t)f); }  // RNE
+
+// Streaming (non-temporal) loads for data that is read exactly once.
+__device__ __forceinline__ u32x4 load_nt(const u32x4* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ uint32_t load_nt(const uint32_t* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ uint16_t load_nt(const uint16_t* p) { return __builtin_nontemporal_load(p); }
+
+// fp32 += a.x*b.x + a.y*b.y (v_dot2_f32_f16)
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(as_h2(a), as_h2(b), c, false);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Sum within each aligned group of 16 lanes (a DPP row); every lane of the
+// group ends up holding the group's sum.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_mov<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_mov<0x124>(v);  // row_ror:4
+    v += dpp_mov<0x128>(v);  // row_ror:8
+    return v;
+}
+// Sum over the 64 lanes of the wave; the result is wave-uniform.
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+// Sum within aligned groups of LP lanes (LP = 8, 16 or 32).
+template <int LP>
+__device__ __forceinline__ float group_sum(float v) {
+    static_assert(LP == 8 || LP == 16 || LP == 32, "unsupported group width");
+    v += dpp_mov<0xB1>(v);
+    v += dpp_mov<0x4E>(v);
+    if (LP == 8) {
+        v += dpp_mov<0x141>(v);  // row_half_mirror: quads 0<->1 inside each 8 lanes
+    } else {
+        v += dpp_mov<0x124>(v);
+        v += dpp_mov<0x128>(v);
+        if (LP == 32) v += __shfl_xor(v, 16);
+    }
+    return v;
+}
+
+#endif  // __HIPCC__

@@ -1,0 +1,463 @@
+// The fp16 side of batch-1 decode on gfx950: embedding gather, RMSNorm, RoPE,
+// KV-cache attention, the fp16 classifier matrix-vector product and the greedy
+// sampler.  Arithmetic and rounding points follow the reference kernels cited
+// at each entry point; launch geometry and data movement are this library's.
+#include "common.hpp"
+
+namespace {
+
+// ------------------------------------------------------------------ embed
+__global__ __launch_bounds__(256) void embed_kernel(uint16_t* x, const uint16_t* table, int dim, const int* tokens,
+                                                    const int* pPos) {
+    const int token = tokens[*pPos];
+    const u32x4* src = reinterpret_cast<const u32x4*>(table + (size_t)token * dim);
+    u32x4* dst = reinterpret_cast<u32x4*>(x);
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < (dim >> 3)) dst[i] = src[i];
+}
+
+// ------------------------------------------------------------------ rmsnorm
+// One workgroup of 1024 (the vector is a few KB): fp32 sum of squares,
+// ss = 1/sqrt(ss/size + 1e-5), o = half(x * (ss * w)).
+__global__ __launch_bounds__(1024) void rmsnorm_kernel(uint16_t* o, const uint16_t* x, const uint16_t* weight, int size) {
+    __shared__ float red[16];
+    __shared__ float shared_ss;
+    const int tid = threadIdx.x;
+    float part = 0.0f;
+    for (int i = tid; i < size; i += 1024) {
+        const float v = half_bits_to_float(x[i]);
+        part = fmaf(v, v, part);
+    }
+    part = wave_sum(part);
+    if ((tid & 63) == 0) red[tid >> 6] = part;
+    __syncthreads();
+    if (tid == 0) {
+        float ss = 0.0f;
+        for (int w = 0; w < 16; w++) ss += red[w];
+        ss /= (float)size;
+        ss += 1e-5f;
+        shared_ss = 1.0f / sqrtf(ss);
+    }
+    __syncthreads();
+    const float ss = shared_ss;
+    for (int i = tid; i < size; i += 1024) {
+        const float v = half_bits_to_float(x[i]);
+        o[i] = float_to_half_bits(v * (ss * half_bits_to_float(weight[i])));
+    }
+}
+
+// ------------------------------------------------------------------ rope
+// One workgroup per head, one thread per pair (i, i + head/2).
+__global__ void rope_kernel(uint16_t* sq, uint16_t* sk_base, int num_kv_heads, int head_size, const int* pPos, int loff,
+                            float rope_theta) {
+    const int pos = *pPos;
+    const int h = blockIdx.x;
+    const int i = threadIdx.x;
+    const int half_size = head_size >> 1;
+    const int head_dim = (i * 2) % head_size;
+    const float freq = 1.0f / powf(rope_theta, head_dim / (float)head_size);
+    const float val = pos * freq;
+    const float fcr = cosf(val);
+    const float fci = sinf(val);
+    uint16_t* q = sq + (size_t)h * head_size;
+    const float q0 = half_bits_to_float(q[i]);
+    const float q1 = half_bits_to_float(q[i + half_size]);
+    q[i] = float_to_half_bits(q0 * fcr - q1 * fci);
+    q[i + half_size] = float_to_half_bits(q0 * fci + q1 * fcr);
+    if (h < num_kv_heads) {
+        uint16_t* k = sk_base + (size_t)loff + (size_t)pos * num_kv_heads * head_size + (size_t)h * head_size;
+        const float k0 = half_bits_to_float(k[i]);
+        const float k1 = half_bits_to_float(k[i + half_size]);
+        k[i] = float_to_half_bits(k0 * fcr - k1 * fci);
+        k[i + half_size] = float_to_half_bits(k0 * fci + k1 * fcr);
+    }
+}
+
+// ------------------------------------------------------------------ attention
+// Pass 1: scores.  LP = head_size/8 lanes cover one cache row of a head
+// (16 bytes each); a wave covers 64/LP positions per load and a workgroup of
+// 4 waves covers 64 positions.  att[h*(pos+1) + t] = half(dot(K[t], q) / sqrt(head)).
+template <int LP>
+__global__ __launch_bounds__(256) void attn_scores_kernel(uint16_t* att, const uint16_t* q, const uint16_t* key_cache,
+                                                          int head_size, int kv_mul, int row_stride, float alpha,
+                                                          const int* pPos) {
+    const int size = *pPos + 1;
+    const int t0 = blockIdx.x * 64;
+    if (t0 >= size) return;
+    const int h = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    constexpr int PW = 64 / LP;  // positions per wave-load
+    const int j = lane % LP;     // which 8 halves of the head
+    const int pr = lane / LP;
+    const u32x4 qv = *reinterpret_cast<const u32x4*>(q + (size_t)h * head_size + j * 8);
+    const uint16_t* kh = key_cache + (size_t)(h / kv_mul) * head_size + j * 8;
+    uint16_t* a = att + (size_t)h * size;
+    constexpr int ITERS = 16 / PW;  // 16 positions per wave
+    u32x4 kv[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int t = t0 + wave * 16 + it * PW + pr;
+        if (t < size) kv[it] = *reinterpret_cast<const u32x4*>(kh + (size_t)t * row_stride);
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int t = t0 + wave * 16 + it * PW + pr;
+        float s = 0.0f;
+        if (t < size) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) s = dot2(kv[it][i], qv[i], s);
+        }
+        s = group_sum<LP>(s);
+        if (j == 0 && t < size) a[t] = float_to_half_bits(s * alpha);
+    }
+}
+
+// Pass 2: softmax statistics (recomputed by every workgroup of a head from the
+// fp16 scores: a few KB), probabilities rounded to fp16 as the reference
+// does, and P.V over this workgroup's slice of positions.  With more than one
+// split the per-split partial sums are combined, in split order, by the last
+// workgroup of the head to arrive.
+template <int LP>
+__global__ __launch_bounds__(256) void attn_softmax_pv_kernel(uint16_t* output, const uint16_t* att,
+                                                              const uint16_t* value_cache, int head_size, int kv_mul,
+                                                              int row_stride, const int* pPos, float* partial,
+                                                              unsigned int* counter) {
+    __shared__ float red[4];
+    __shared__ float acc_lds[4][kAttnMaxHeadSize];
+    __shared__ unsigned int arrival;
+    const int size = *pPos + 1;
+    const int h = blockIdx.y;
+    const int nsplit = gridDim.x;
+    const int split = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const uint16_t* a = att + (size_t)h * size;
+
+    // max (the reference seeds idle threads of its 1024-thread block with 0)
+    float m = (size < 1024) ? 0.0f : -INFINITY;
+    for (int t = tid; t < size; t += 256) m = fmaxf(m, half_bits_to_float(a[t]));
+    m = wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float sum = 0.0f;
+    for (int t = tid; t < size; t += 256) sum += expf(half_bits_to_float(a[t]) - m);
+    sum = wave_sum(sum);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    sum = (red[0] + red[1]) + (red[2] + red[3]);
+
+    // this workgroup's positions
+    const int per = (size + nsplit - 1) / nsplit;
+    const int tb = split * per;
+    const int te = min(size, tb + per);
+    constexpr int PW = 64 / LP;
+    const int j = lane % LP;
+    const int pr = lane / LP;
+    const uint16_t* vh = value_cache + (size_t)(h / kv_mul) * head_size + j * 8;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.0f;
+    for (int t = tb + wave * PW + pr; t < te; t += 4 * PW) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+        const float e = expf(half_bits_to_float(a[t]) - m);
+        const float p = half_bits_to_float(float_to_half_bits(e / sum));  // probability rounded to fp16
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const h16x2 hv = as_h2(v[i]);
+            acc[2 * i] = fmaf((float)hv[0], p, acc[2 * i]);
+            acc[2 * i + 1] = fmaf((float)hv[1], p, acc[2 * i + 1]);
+        }
+    }
+    // combine the PW position groups of the wave, then the 4 waves
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        for (int off = LP; off < 64; off <<= 1) acc[i] += __shfl_xor(acc[i], off);
+    }
+    if (pr == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc_lds[wave][j * 8 + i] = acc[i];
+    }
+    __syncthreads();
+    float total = 0.0f;
+    if (tid < head_size) total = (acc_lds[0][tid] + acc_lds[1][tid]) + (acc_lds[2][tid] + acc_lds[3][tid]);
+
+    if (nsplit == 1) {
+        if (tid < head_size) output[(size_t)h * head_size + tid] = float_to_half_bits(total);
+        return;
+    }
+    float* my = partial + ((size_t)h * kAttnMaxSplits + split) * kAttnMaxHeadSize;
+    if (tid < head_size) my[tid] = total;
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) arrival = atomicAdd(&counter[h], 1u);
+    __syncthreads();
+    if (arrival == (unsigned int)(nsplit - 1)) {
+        __threadfence();
+        if (tid < head_size) {
+            const float* ph = partial + (size_t)h * kAttnMaxSplits * kAttnMaxHeadSize;
+            float s = 0.0f;
+            for (int sp = 0; sp < nsplit; sp++) s += ph[(size_t)sp * kAttnMaxHeadSize + tid];
+            output[(size_t)h * head_size + tid] = float_to_half_bits(s);
+        }
+        if (tid == 0) counter[h] = 0;  // ready for the next launch
+    }
+}
+
+// ------------------------------------------------------------------ fp16 matvec
+// out[r] = half(sum_j w[r*n + j] * x[j]).  x staged in LDS in natural order;
+// a lane owns the same 16-byte column slices for the R rows of its wave.
+template <int R, bool NORM>
+__global__ __launch_bounds__(256) void gemv_f16_kernel(uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
+                                                       const uint16_t* norm_w, uint16_t* norm_out) {
+    extern __shared__ u32x4 xs[];
+    __shared__ float red[4];
+    const int tid = threadIdx.x;
+    const int n8 = n >> 3;
+    const u32x4* xg = reinterpret_cast<const u32x4*>(x);
+    float ss = 0.0f;
+    if (NORM) {
+        float part = 0.0f;
+        for (int e = tid; e < n8; e += 256) {
+            const u32x4 v = xg[e];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const h16x2 hh = as_h2(v[i]);
+                const float a = (float)hh[0], b = (float)hh[1];
+                part = fmaf(a, a, part);
+                part = fmaf(b, b, part);
+            }
+        }
+        part = wave_sum(part);
+        if ((tid & 63) == 0) red[tid >> 6] = part;
+        __syncthreads();
+        ss = (red[0] + red[1]) + (red[2] + red[3]);
+        ss /= (float)n;
+        ss += 1e-5f;
+        ss = 1.0f / sqrtf(ss);
+    }
+    const bool store_norm = NORM && norm_out != nullptr && blockIdx.x == 0;
+    for (int e = tid; e < n8; e += 256) {
+        u32x4 v = xg[e];
+        if (NORM) {
+            const u32x4 wv = reinterpret_cast<const u32x4*>(norm_w)[e];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const h16x2 hh = as_h2(v[i]);
+                const h16x2 hw = as_h2(wv[i]);
+                h16x2 o;
+                o[0] = (h16_t)((float)hh[0] * (ss * (float)hw[0]));
+                o[1] = (h16_t)((float)hh[1] * (ss * (float)hw[1]));
+                v[i] = as_u32(o);
+            }
+        }
+        xs[e] = v;
+    }
+    __syncthreads();
+    // norm_out must not alias x: other workgroups may still be reading x.
+    if (store_norm) {
+        for (int e = tid; e < n8; e += 256) reinterpret_cast<u32x4*>(norm_out)[e] = xs[e];
+    }
+
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int row0 = (blockIdx.x * 4 + wave) * R;
+    if (row0 >= d) return;
+    const u32x4* wrow[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) wrow[r] = reinterpret_cast<const u32x4*>(w + (size_t)min(row0 + r, d - 1) * n);
+    float sum[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) sum[r] = 0.0f;
+
+    u32x4 a[R], b[R];
+    if (lane < n8) {
+#pragma unroll
+        for (int r = 0; r < R; r++) a[r] = load_nt(wrow[r] + lane);
+    }
+    for (int c = lane; c < n8 + lane; c += 128) {
+        const int c1 = c + 64, c2 = c + 128;
+        if (c1 < n8) {
+#pragma unroll
+            for (int r = 0; r < R; r++) b[r] = load_nt(wrow[r] + c1);
+        }
+        if (c < n8) {
+            const u32x4 xv = xs[c];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) sum[r] = dot2(a[r][i], xv[i], sum[r]);
+        }
+        if (c2 < n8) {
+#pragma unroll
+            for (int r = 0; r < R; r++) a[r] = load_nt(wrow[r] + c2);
+        }
+        if (c1 < n8) {
+            const u32x4 xv = xs[c1];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) sum[r] = dot2(b[r][i], xv[i], sum[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) sum[r] = wave_sum(sum[r]);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (row0 + r < d) out[row0 + r] = float_to_half_bits(sum[r]);
+    }
+}
+
+// ------------------------------------------------------------------ argmax
+// One workgroup of 1024: per-thread strided scan keeping the first maximum,
+// then (value, index) reductions that prefer the lower index on equal values.
+__global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* x, int size, int* result, volatile int* pPos,
+                                                      int* pPosGpu, int write_token) {
+    __shared__ float red_v[16];
+    __shared__ int red_i[16];
+    const int tid = threadIdx.x;
+    float best = -INFINITY;
+    int best_i = 0x7FFFFFFF;
+    for (int i = tid; i < size; i += 1024) {
+        const float v = half_bits_to_float(x[i]);
+        if (v > best) {
+            best = v;
+            best_i = i;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off);
+        const int oi = __shfl_xor(best_i, off);
+        if (ov > best || (ov == best && oi < best_i)) {
+            best = ov;
+            best_i = oi;
+        }
+    }
+    if ((tid & 63) == 0) {
+        red_v[tid >> 6] = best;
+        red_i[tid >> 6] = best_i;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 16; w++) {
+            if (red_v[w] > best || (red_v[w] == best && red_i[w] < best_i)) {
+                best = red_v[w];
+                best_i = red_i[w];
+            }
+        }
+        if (best_i == 0x7FFFFFFF) best_i = 0;  // nothing compared greater than -inf (all NaN / -inf)
+        int token_pos = *pPosGpu;
+        token_pos++;
+        if (write_token) result[token_pos] = best_i;
+        *pPos = token_pos;
+        *pPosGpu = token_pos;
+    }
+}
+
+template <int LP>
+int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const uint16_t* key_cache,
+                     const uint16_t* value_cache, uint16_t* att, int num_heads, int head_size, int kv_mul, int max_seq_len,
+                     const int* pos) {
+    const int row_stride = num_heads * head_size / kv_mul;
+    const float alpha = (float)(1.0 / sqrt((double)head_size));
+    hipLaunchKernelGGL((attn_scores_kernel<LP>), dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, ctx->stream, att, q,
+                       key_cache, head_size, kv_mul, row_stride, alpha, pos);
+    if (int r = awq_check_launch("attn_scores")) return r;
+    int nsplit = div_up(max_seq_len, 256);
+    if (nsplit > kAttnMaxSplits) nsplit = kAttnMaxSplits;
+    if (nsplit < 1) nsplit = 1;
+    hipLaunchKernelGGL((attn_softmax_pv_kernel<LP>), dim3(nsplit, num_heads), dim3(256), 0, ctx->stream, output, att,
+                       value_cache, head_size, kv_mul, row_stride, pos, ctx->attn_partial, ctx->attn_counter);
+    return awq_check_launch("attn_softmax_pv");
+}
+
+}  // namespace
+
+// Internal: fp16 matvec with optional fused RMSNorm of x (norm_out must not alias x).
+int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
+                          const uint16_t* norm_w, uint16_t* norm_out) {
+    constexpr int R = 4;
+    const dim3 grid(div_up(d, 4 * R));
+    const size_t lds = (size_t)n * 2;
+    if (norm_w)
+        hipLaunchKernelGGL((gemv_f16_kernel<R, true>), grid, dim3(256), lds, ctx->stream, out, x, w, n, d, norm_w, norm_out);
+    else
+        hipLaunchKernelGGL((gemv_f16_kernel<R, false>), grid, dim3(256), lds, ctx->stream, out, x, w, n, d, norm_w, norm_out);
+    return awq_check_launch("gemv_f16");
+}
+
+extern "C" {
+
+int awq_embed(awq_ctx* ctx, uint16_t* x, const uint16_t* table, int dim, const int* tokens, const int* pos) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(x && table && tokens && pos, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(dim > 0 && (dim & 7) == 0, AWQ_ERR_SHAPE, "dim must be a positive multiple of 8");
+    hipLaunchKernelGGL(embed_kernel, dim3(div_up(dim >> 3, 256)), dim3(256), 0, ctx->stream, x, table, dim, tokens, pos);
+    return awq_check_launch("embed");
+}
+
+int awq_rmsnorm(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const uint16_t* weight, int size) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(o && x && weight, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(size > 0, AWQ_ERR_SHAPE, "size must be positive");
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(1024), 0, ctx->stream, o, x, weight, size);
+    return awq_check_launch("rmsnorm");
+}
+
+int awq_rope(awq_ctx* ctx, uint16_t* q, uint16_t* k, int num_heads, int num_kv_heads, int head_size, const int* pos, int loff,
+             float rope_theta) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(q && k && pos, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(num_heads > 0 && num_kv_heads >= 0 && num_kv_heads <= num_heads, AWQ_ERR_SHAPE, "bad head counts");
+    AWQ_REQUIRE(head_size >= 2 && (head_size & 1) == 0 && head_size <= 2048, AWQ_ERR_SHAPE, "head_size must be even, <= 2048");
+    AWQ_REQUIRE(loff >= 0, AWQ_ERR_ARG, "loff must be >= 0");
+    hipLaunchKernelGGL(rope_kernel, dim3(num_heads), dim3(head_size / 2), 0, ctx->stream, q, k, num_kv_heads, head_size, pos,
+                       loff, rope_theta);
+    return awq_check_launch("rope");
+}
+
+int awq_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const uint16_t* key_cache, const uint16_t* value_cache,
+                  uint16_t* att, int num_heads, int head_size, int kv_mul, int max_seq_len, const int* pos) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(output && q && key_cache && value_cache && att && pos, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(num_heads > 0 && num_heads <= kAttnMaxHeads, AWQ_ERR_SHAPE, "num_heads out of range");
+    AWQ_REQUIRE(kv_mul > 0 && num_heads % kv_mul == 0, AWQ_ERR_SHAPE, "kv_mul must divide num_heads");
+    AWQ_REQUIRE(max_seq_len > 0, AWQ_ERR_SHAPE, "max_seq_len must be positive");
+    switch (head_size) {
+        case 64:
+            return launch_attention<8>(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos);
+        case 128:
+            return launch_attention<16>(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos);
+        case 256:
+            return launch_attention<32>(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos);
+        default:
+            awq_set_error("awq_attention: head_size %d unsupported (64, 128 or 256)", head_size);
+            return AWQ_ERR_SHAPE;
+    }
+}
+
+int awq_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d) {
+    if (int r = awq_bind(ctx)) return r;
+    if (n <= 0 || d <= 0 || (n & 7) || (d & 7)) {  // llama2_q4.cu:358
+        awq_set_error("unsupported matmul size n=%d d=%d (both must be positive multiples of 8)", n, d);
+        return AWQ_ERR_SHAPE;
+    }
+    AWQ_REQUIRE(n <= kMaxStagedK, AWQ_ERR_SHAPE, "n exceeds the activations staged in LDS");
+    AWQ_REQUIRE(out && x && w, AWQ_ERR_ARG, "null pointer");
+    return awq_launch_matvec_f16(ctx, out, x, w, n, d, nullptr, nullptr);
+}
+
+int awq_argmax_advance(awq_ctx* ctx, const uint16_t* logits, int size, int* tokens, volatile int* pos_host, int* pos_dev,
+                       int write_token) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(logits && tokens && pos_host && pos_dev, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(size > 0, AWQ_ERR_SHAPE, "size must be positive");
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, ctx->stream, logits, size, tokens, pos_host, pos_dev, write_token);
+    return awq_check_launch("argmax");
+}
+
+}  // extern "C"

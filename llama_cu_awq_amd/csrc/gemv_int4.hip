@@ -1,0 +1,410 @@
+// AWQ int4 group-128 matrix-vector kernels for gfx950 (wave64).
+//
+// What they compute is the reference's mat_vec_kernel_int4 family
+// (gpu_kernels.h:179-283): per output row n,
+//     sum_k (q[n,k] - z[n,k/128]) * s[n,k/128] * x[k]   in fp32,
+// followed by one of the epilogues (plain store, KV-cache row store, fused
+// residual add, SiLU(gate)*up).
+//
+// How: a workgroup of 4 waves stages the activation vector once in LDS
+// (optionally applying RMSNorm on the way in), pre-permuted so that a lane's
+// 32 consecutive K elements (one 16-byte load of packed weights, the same lane
+// ownership as the reference's uint4 load) meet their activations as packed
+// fp16 pairs.  Each wave owns R consecutive rows and walks the row in passes
+// of 64 x 16 bytes, with the next pass's loads issued before the current pass
+// is consumed; a lane keeps its activations in registers across the R rows.
+// Nibbles become fp16 integers with the 0x6400 mantissa trick, the zero point
+// is subtracted exactly in fp16, products are accumulated in fp32 by
+// v_dot2_f32_f16, and the group scale is applied once per 32 elements in fp32.
+#include "common.hpp"
+
+namespace {
+
+struct Int4Mat {
+    const uint32_t* w;
+    const uint32_t* z;
+    const uint16_t* s;
+};
+
+struct GemvParams {
+    Int4Mat m[3];            // [0] for the single form; q,k,v; gate,up
+    uint16_t* out[3];
+    const uint16_t* x;
+    const uint16_t* norm_w;  // RMSNorm weights when the norm is fused into staging
+    uint16_t* norm_out;      // optional: block 0 also stores the normalised vector here
+    int K, N;
+    int C;                   // 32-element chunks per row = ceil(K/32)
+    int pzh, sh;             // zeros dwords / scale halves per row
+    int accum;
+    float inv_gpu_count;
+    int loff[3];             // -1: none; else out += loff + *pos * N
+    const int* pos;
+};
+
+enum { KIND_SINGLE = 0, KIND_QKV = 1, KIND_FFN = 2 };
+
+// Sum over 32 consecutive K elements of (q - z) * x, exact products, fp32 sum.
+// w: 4 dwords of 8 nibbles; xq[qi]: the 8 activations of dword qi as pairs
+// (0,4) (1,5) (2,6) (3,7).
+__device__ __forceinline__ float chunk_dot(const u32x4 w, const uint32_t z, const u32x4 (&xq)[4]) {
+    // fp16 constants: -(1024 + z) and -(64 + z), both exactly representable
+    const h16x2 zlo = as_h2(0xE400E400u | (z * 0x00010001u));
+    const h16x2 zhi = as_h2(0xD400D400u | (z * 0x00100010u));
+    const h16x2 sixteenth = {(h16_t)0.0625f, (h16_t)0.0625f};
+    float acc = 0.0f;
+#pragma unroll
+    for (int qi = 0; qi < 4; qi++) {
+        const uint32_t d = w[qi];
+        const uint32_t d8 = d >> 8;
+        // 0x6400 | n  == 1024 + n ;  0x6400 | (n << 4) == 1024 + 16 n   (fp16, exact)
+        h16x2 t0 = as_h2((d & 0x000F000Fu) | 0x64006400u) + zlo;                                     // q0-z, q4-z
+        h16x2 t1 = __builtin_elementwise_fma(as_h2((d & 0x00F000F0u) | 0x64006400u), sixteenth, zhi);   // q1-z, q5-z
+        h16x2 t2 = as_h2((d8 & 0x000F000Fu) | 0x64006400u) + zlo;                                    // q2-z, q6-z
+        h16x2 t3 = __builtin_elementwise_fma(as_h2((d8 & 0x00F000F0u) | 0x64006400u), sixteenth, zhi);  // q3-z, q7-z
+        acc = __builtin_amdgcn_fdot2(t0, as_h2(xq[qi][0]), acc, false);
+        acc = __builtin_amdgcn_fdot2(t1, as_h2(xq[qi][1]), acc, false);
+        acc = __builtin_amdgcn_fdot2(t2, as_h2(xq[qi][2]), acc, false);
+        acc = __builtin_amdgcn_fdot2(t3, as_h2(xq[qi][3]), acc, false);
+    }
+    return acc;
+}
+
+template <int NS>
+struct Stage {
+    u32x4 w[NS];
+    uint32_t zw[NS];
+    uint16_t s[NS];
+};
+
+template <int NS>
+__device__ __forceinline__ void load_stage(Stage<NS>& st, const uint32_t* const (&wrow)[NS],
+                                           const uint32_t* const (&zrow)[NS], const uint16_t* const (&srow)[NS], int c,
+                                           int C) {
+    if (c < C) {
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            st.w[i] = load_nt(reinterpret_cast<const u32x4*>(wrow[i]) + c);
+            st.zw[i] = zrow[i][c >> 5];
+            st.s[i] = srow[i][c >> 2];
+        }
+    }
+}
+
+template <int NS>
+__device__ __forceinline__ void consume_stage(const Stage<NS>& st, const u32x4* xs, int c, int C, float (&sum)[NS]) {
+    if (c < C) {
+        u32x4 xq[4];
+#pragma unroll
+        for (int qi = 0; qi < 4; qi++) xq[qi] = xs[qi * C + c];
+        const int zshift = ((c >> 2) & 7) * 4;
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            const uint32_t z = (st.zw[i] >> zshift) & 0xFu;
+            const float acc = chunk_dot(st.w[i], z, xq);
+            sum[i] = fmaf(half_bits_to_float(st.s[i]), acc, sum[i]);
+        }
+    }
+}
+
+// Stage x (K halves) into LDS as u32x4 words laid out [qi][chunk], each holding
+// the 8 activations of dword qi of that chunk as pairs (0,4)(1,5)(2,6)(3,7);
+// elements in [K, 32*C) are zero.  With NORM the vector is RMS-normalised on
+// the way in with the reference's arithmetic (gpu_kernels.h:72-105):
+// o = half(x * (rsqrt(mean(x^2) + 1e-5) * w)).
+template <bool NORM>
+__device__ __forceinline__ void stage_x(u32x4* xs, const GemvParams& p, float* red) {
+    const int tid = threadIdx.x;
+    const int n8 = p.K >> 3;  // 8-half pieces of real data
+    const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
+    float ss = 0.0f;
+    if (NORM) {
+        float part = 0.0f;
+        for (int e = tid; e < n8; e += 256) {
+            const u32x4 v = xg[e];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const h16x2 h = as_h2(v[i]);
+                const float a = (float)h[0], b = (float)h[1];
+                part = fmaf(a, a, part);
+                part = fmaf(b, b, part);
+            }
+        }
+        part = wave_sum(part);
+        if ((tid & 63) == 0) red[tid >> 6] = part;
+        __syncthreads();
+        ss = (red[0] + red[1]) + (red[2] + red[3]);
+        ss /= (float)p.K;
+        ss += 1e-5f;
+        ss = 1.0f / sqrtf(ss);
+    }
+    const u32x4* wg = reinterpret_cast<const u32x4*>(p.norm_w);
+    u32x4* og = reinterpret_cast<u32x4*>(p.norm_out);
+    const bool store_norm = NORM && og != nullptr && blockIdx.x == 0 && blockIdx.y == 0;
+    for (int e = tid; e < p.C * 4; e += 256) {
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (e < n8) {
+            v = xg[e];
+            if (NORM) {
+                const u32x4 wv = wg[e];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const h16x2 h = as_h2(v[i]);
+                    const h16x2 hw = as_h2(wv[i]);
+                    h16x2 o;
+                    o[0] = (h16_t)((float)h[0] * (ss * (float)hw[0]));
+                    o[1] = (h16_t)((float)h[1] * (ss * (float)hw[1]));
+                    v[i] = as_u32(o);
+                }
+                if (store_norm) og[e] = v;
+            }
+        }
+        // v holds halves h0..h7 as (h0,h1)(h2,h3)(h4,h5)(h6,h7) -> (h0,h4)(h1,h5)(h2,h6)(h3,h7)
+        u32x4 o;
+        o[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
+        o[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
+        o[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
+        o[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
+        xs[(e & 3) * p.C + (e >> 2)] = o;
+    }
+    __syncthreads();
+}
+
+template <int R, int KIND, bool NORM>
+__global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
+    extern __shared__ u32x4 xs[];
+    __shared__ float red[4];
+    stage_x<NORM>(xs, p, red);
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int C = p.C;
+    const int pwh = C * 4;
+    const int which = (KIND == KIND_QKV) ? blockIdx.y : 0;
+    const int row0 = (blockIdx.x * 4 + wave) * R;
+    if (row0 >= p.N) return;
+
+    constexpr int NS = (KIND == KIND_FFN) ? 2 * R : R;
+    const uint32_t* wrow[NS];
+    const uint32_t* zrow[NS];
+    const uint16_t* srow[NS];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = min(row0 + r, p.N - 1);  // rows past N are recomputed and not stored
+        if (KIND == KIND_FFN) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                wrow[2 * r + j] = p.m[j].w + (size_t)row * pwh;
+                zrow[2 * r + j] = p.m[j].z + (size_t)row * p.pzh;
+                srow[2 * r + j] = p.m[j].s + (size_t)row * p.sh;
+            }
+        } else {
+            const Int4Mat m = (KIND == KIND_QKV) ? (which == 0 ? p.m[0] : (which == 1 ? p.m[1] : p.m[2])) : p.m[0];
+            wrow[r] = m.w + (size_t)row * pwh;
+            zrow[r] = m.z + (size_t)row * p.pzh;
+            srow[r] = m.s + (size_t)row * p.sh;
+        }
+    }
+
+    float sum[NS];
+#pragma unroll
+    for (int i = 0; i < NS; i++) sum[i] = 0.0f;
+
+    Stage<NS> a, b;
+    load_stage<NS>(a, wrow, zrow, srow, lane, C);
+    for (int c = lane; c < C + lane; c += 128) {  // wave-uniform trip count
+        const int c1 = c + 64;
+        load_stage<NS>(b, wrow, zrow, srow, c1, C);
+        consume_stage<NS>(a, xs, c, C, sum);
+        load_stage<NS>(a, wrow, zrow, srow, c1 + 64, C);
+        consume_stage<NS>(b, xs, c1, C, sum);
+    }
+
+#pragma unroll
+    for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]);
+
+    if (lane == 0) {
+        uint16_t* out = (KIND == KIND_QKV) ? (which == 0 ? p.out[0] : (which == 1 ? p.out[1] : p.out[2])) : p.out[0];
+        const int loff = (KIND == KIND_QKV) ? (which == 0 ? p.loff[0] : (which == 1 ? p.loff[1] : p.loff[2])) : p.loff[0];
+        if (loff != -1) out += (size_t)loff + (size_t)(*p.pos) * p.N;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = row0 + r;
+            if (row < p.N) {
+                float v;
+                if (KIND == KIND_FFN) {
+                    // gate = stream 2r, up = stream 2r+1 (gpu_kernels.h:276-281)
+                    float g = sum[2 * r];
+                    g *= 1.0f / (1.0f + expf(-g));
+                    v = g * sum[2 * r + 1];
+                } else {
+                    v = sum[r];
+                    if (KIND == KIND_SINGLE && p.accum) v += half_bits_to_float(out[row]) * p.inv_gpu_count;
+                }
+                out[row] = float_to_half_bits(v);
+            }
+        }
+    }
+}
+
+// out[n*K + k] = half_rne((q - z) * s): exact fp32 product, one rounding.
+__global__ __launch_bounds__(256) void dequant_kernel(uint16_t* out, Int4Mat m, int K, int N, int pwh, int pzh, int sh) {
+    const size_t total8 = (size_t)N * (K >> 3);
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total8; e += (size_t)gridDim.x * 256) {
+        const int n = (int)(e / (size_t)(K >> 3));
+        const int k8 = (int)(e % (size_t)(K >> 3));
+        const int g = k8 >> 4;
+        uint32_t d = m.w[(size_t)n * pwh + k8];
+        const float z = (float)((m.z[(size_t)n * pzh + (g >> 3)] >> (4 * (g & 7))) & 0xFu);
+        const float s = half_bits_to_float(m.s[(size_t)n * sh + g]);
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float w0 = ((float)(d & 0xFu) - z) * s;
+            const float w1 = ((float)((d >> 4) & 0xFu) - z) * s;
+            d >>= 8;
+            o[i] = (uint32_t)float_to_half_bits(w0) | ((uint32_t)float_to_half_bits(w1) << 16);
+        }
+        *reinterpret_cast<u32x4*>(out + (size_t)n * K + (size_t)k8 * 8) = o;
+    }
+}
+
+int check_shape(int K, int N) {
+    // llama2_q4.cu:368: "Unsupported matmul size"
+    if (K <= 0 || N <= 0 || (K & 7) || (N & 7)) {
+        awq_set_error("unsupported matmul size K=%d N=%d (both must be positive multiples of 8)", K, N);
+        return AWQ_ERR_SHAPE;
+    }
+    if (K > kMaxStagedK) {
+        awq_set_error("K=%d exceeds the %d activations the kernels stage in LDS", K, kMaxStagedK);
+        return AWQ_ERR_SHAPE;
+    }
+    return AWQ_OK;
+}
+
+void fill_common(GemvParams& p, const uint16_t* x, int K, int N) {
+    p.x = x;
+    p.norm_w = nullptr;
+    p.norm_out = nullptr;
+    p.K = K;
+    p.N = N;
+    p.C = div_up(K, 32);
+    p.pzh = packed_zeros_height(K);
+    p.sh = scales_height(K);
+    p.accum = 0;
+    p.inv_gpu_count = 1.0f;
+    p.loff[0] = p.loff[1] = p.loff[2] = -1;
+    p.pos = nullptr;
+}
+
+Int4Mat to_mat(const awq_qweight* w) { return Int4Mat{w->weight, w->zeros, w->scales}; }
+
+bool qw_ok(const awq_qweight* w) { return w && w->weight && w->zeros && w->scales; }
+
+template <int R, int KIND>
+int launch(awq_ctx* ctx, const GemvParams& p, int grid_y, const char* what) {
+    const dim3 grid(div_up(p.N, 4 * R), grid_y);
+    const size_t lds = (size_t)p.C * 64;
+    if (p.norm_w)
+        hipLaunchKernelGGL((gemv_int4_kernel<R, KIND, true>), grid, dim3(256), lds, ctx->stream, p);
+    else
+        hipLaunchKernelGGL((gemv_int4_kernel<R, KIND, false>), grid, dim3(256), lds, ctx->stream, p);
+    return awq_check_launch(what);
+}
+
+}  // namespace
+
+// Internal launchers shared with the fused schedule (norm_w != nullptr fuses
+// RMSNorm into the staging of x; norm_out optionally receives the normalised vector).
+int awq_launch_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* w, int K, int N, int accum,
+                           int gpu_count, int loff, const int* pos, const uint16_t* norm_w, uint16_t* norm_out) {
+    GemvParams p;
+    fill_common(p, x, K, N);
+    p.m[0] = to_mat(w);
+    p.out[0] = out;
+    p.accum = accum;
+    p.inv_gpu_count = 1.0f / (float)gpu_count;
+    p.loff[0] = loff;
+    p.pos = pos;
+    p.norm_w = norm_w;
+    p.norm_out = norm_out;
+    // 2 rows per wave keep >= 2 workgroups per CU busy at N = 4096; 4 rows amortise staging on big N
+    if (N >= 8192) return launch<4, KIND_SINGLE>(ctx, p, 1, "gemv_int4");
+    return launch<2, KIND_SINGLE>(ctx, p, 1, "gemv_int4");
+}
+
+int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
+                   const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw, int K, int N, int loff,
+                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out) {
+    GemvParams p;
+    fill_common(p, x, K, N);
+    p.m[0] = to_mat(qw);
+    p.m[1] = to_mat(kw);
+    p.m[2] = to_mat(vw);
+    p.out[0] = q;
+    p.out[1] = key_cache;
+    p.out[2] = value_cache;
+    p.loff[1] = loff;
+    p.loff[2] = loff;
+    p.pos = pos;
+    p.norm_w = norm_w;
+    p.norm_out = norm_out;
+    return launch<4, KIND_QKV>(ctx, p, 3, "qkv_matvec");
+}
+
+int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w, const awq_qweight* up_w, int K,
+                   int N, const uint16_t* norm_w, uint16_t* norm_out) {
+    GemvParams p;
+    fill_common(p, x, K, N);
+    p.m[0] = to_mat(gate_w);
+    p.m[1] = to_mat(up_w);
+    p.out[0] = out;
+    p.norm_w = norm_w;
+    p.norm_out = norm_out;
+    return launch<2, KIND_FFN>(ctx, p, 1, "ffn_matvec_silu");
+}
+
+extern "C" {
+
+int awq_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* w, int K, int N, int accum,
+                    int gpu_count, int loff, const int* pos) {
+    if (int r = awq_bind(ctx)) return r;
+    if (int r = check_shape(K, N)) return r;
+    AWQ_REQUIRE(out && x && qw_ok(w), AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(gpu_count >= 1, AWQ_ERR_ARG, "gpu_count must be >= 1");
+    AWQ_REQUIRE(loff == -1 || (loff >= 0 && pos), AWQ_ERR_ARG, "loff needs a position pointer");
+    return awq_launch_matvec_int4(ctx, out, x, w, K, N, accum, gpu_count, loff, pos, nullptr, nullptr);
+}
+
+int awq_qkv_matvec(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
+                   const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw, int K, int N, int loff,
+                   const int* pos) {
+    if (int r = awq_bind(ctx)) return r;
+    if (int r = check_shape(K, N)) return r;
+    AWQ_REQUIRE(q && key_cache && value_cache && x && qw_ok(qw) && qw_ok(kw) && qw_ok(vw), AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(loff >= 0 && pos, AWQ_ERR_ARG, "qkv needs loff >= 0 and a position pointer");
+    return awq_launch_qkv(ctx, q, key_cache, value_cache, x, qw, kw, vw, K, N, loff, pos, nullptr, nullptr);
+}
+
+int awq_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w, const awq_qweight* up_w,
+                        int K, int N) {
+    if (int r = awq_bind(ctx)) return r;
+    if (int r = check_shape(K, N)) return r;
+    AWQ_REQUIRE(out && x && qw_ok(gate_w) && qw_ok(up_w), AWQ_ERR_ARG, "null pointer");
+    return awq_launch_ffn(ctx, out, x, gate_w, up_w, K, N, nullptr, nullptr);
+}
+
+int awq_dequant(awq_ctx* ctx, uint16_t* out, const awq_qweight* w, int K, int N) {
+    if (int r = awq_bind(ctx)) return r;
+    if (K <= 0 || N <= 0 || (K & 7) || (N & 7)) {
+        awq_set_error("unsupported matmul size K=%d N=%d", K, N);
+        return AWQ_ERR_SHAPE;
+    }
+    AWQ_REQUIRE(out && qw_ok(w), AWQ_ERR_ARG, "null pointer");
+    const size_t total8 = (size_t)N * (K >> 3);
+    const int grid = (int)((total8 + 255) / 256 < 65536 ? (total8 + 255) / 256 : 65536);
+    hipLaunchKernelGGL(dequant_kernel, dim3(grid), dim3(256), 0, ctx->stream, out, to_mat(w), K, N, packed_weight_height(K),
+                       packed_zeros_height(K), scales_height(K));
+    return awq_check_launch("dequant");
+}
+
+}  // extern "C"

@@ -1,0 +1,165 @@
+// Context, memory, stream and timing entry points of libawq_hip.
+// These replace the reference's direct CUDA runtime calls around its hot path
+// (llama2_q4.cu:62-136 allocation, :249 upload, :685-713 device/stream, :545-600 events).
+#include <stdarg.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "common.hpp"
+
+static std::mutex g_err_mutex;
+static char g_err[1024] = "";
+
+void awq_set_error(const char* fmt, ...) {
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" {
+
+const char* awq_last_error(void) { return g_err; }
+
+static int ctx_init(int device, hipStream_t stream, bool owns, awq_ctx** out) {
+    awq_ctx* c = new awq_ctx();
+    c->device = device;
+    c->stream = stream;
+    c->owns_stream = owns;
+    c->attn_partial = nullptr;
+    c->attn_counter = nullptr;
+    size_t partial_bytes = (size_t)kAttnMaxHeads * kAttnMaxSplits * kAttnMaxHeadSize * sizeof(float);
+    hipError_t e = hipMalloc((void**)&c->attn_partial, partial_bytes);
+    if (e == hipSuccess) e = hipMalloc((void**)&c->attn_counter, kAttnMaxHeads * sizeof(unsigned int));
+    if (e == hipSuccess) e = hipMemset(c->attn_counter, 0, kAttnMaxHeads * sizeof(unsigned int));
+    if (e != hipSuccess) {
+        awq_set_error("context workspace allocation failed: %s", hipGetErrorString(e));
+        if (c->attn_partial) (void)hipFree(c->attn_partial);
+        if (c->attn_counter) (void)hipFree(c->attn_counter);
+        if (owns) (void)hipStreamDestroy(stream);
+        delete c;
+        return AWQ_ERR_HIP;
+    }
+    *out = c;
+    return AWQ_OK;
+}
+
+int awq_ctx_create(int device, awq_ctx** out) {
+    AWQ_REQUIRE(out, AWQ_ERR_ARG, "null out");
+    int count = 0;
+    AWQ_HIP_TRY(hipGetDeviceCount(&count));
+    AWQ_REQUIRE(device >= 0 && device < count, AWQ_ERR_ARG, "no such device");
+    AWQ_HIP_TRY(hipSetDevice(device));
+    hipStream_t s;
+    AWQ_HIP_TRY(hipStreamCreate(&s));  // default priority
+    return ctx_init(device, s, true, out);
+}
+
+int awq_ctx_create_on_stream(int device, void* hip_stream, awq_ctx** out) {
+    AWQ_REQUIRE(out, AWQ_ERR_ARG, "null out");
+    AWQ_HIP_TRY(hipSetDevice(device));
+    return ctx_init(device, (hipStream_t)hip_stream, false, out);
+}
+
+int awq_ctx_destroy(awq_ctx* ctx) {
+    if (int r = awq_bind(ctx)) return r;
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->attn_partial);
+    (void)hipFree(ctx->attn_counter);
+    if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return AWQ_OK;
+}
+
+int awq_stream_sync(awq_ctx* ctx) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return AWQ_OK;
+}
+
+void* awq_ctx_stream(awq_ctx* ctx) { return ctx ? (void*)ctx->stream : nullptr; }
+
+int awq_malloc(awq_ctx* ctx, void** ptr, size_t bytes) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(ptr, AWQ_ERR_ARG, "null ptr");
+    AWQ_HIP_TRY(hipMalloc(ptr, bytes ? bytes : 1));
+    return AWQ_OK;
+}
+
+int awq_free(awq_ctx* ctx, void* ptr) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipFree(ptr));
+    return AWQ_OK;
+}
+
+int awq_malloc_host(awq_ctx* ctx, void** ptr, size_t bytes) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(ptr, AWQ_ERR_ARG, "null ptr");
+    AWQ_HIP_TRY(hipHostMalloc(ptr, bytes ? bytes : 1, hipHostMallocDefault));
+    return AWQ_OK;
+}
+
+int awq_free_host(awq_ctx* ctx, void* ptr) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipHostFree(ptr));
+    return AWQ_OK;
+}
+
+int awq_memcpy_h2d_async(awq_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    return AWQ_OK;
+}
+
+int awq_memcpy_h2d(awq_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    AWQ_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return AWQ_OK;
+}
+
+int awq_memcpy_d2h(awq_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    AWQ_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return AWQ_OK;
+}
+
+int awq_memset_async(awq_ctx* ctx, void* dst, int value, size_t bytes) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipMemsetAsync(dst, value, bytes, ctx->stream));
+    return AWQ_OK;
+}
+
+int awq_event_create(awq_ctx* ctx, void** event) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(event, AWQ_ERR_ARG, "null event");
+    hipEvent_t e;
+    AWQ_HIP_TRY(hipEventCreate(&e));
+    *event = (void*)e;
+    return AWQ_OK;
+}
+
+int awq_event_destroy(awq_ctx* ctx, void* event) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipEventDestroy((hipEvent_t)event));
+    return AWQ_OK;
+}
+
+int awq_event_record(awq_ctx* ctx, void* event) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipEventRecord((hipEvent_t)event, ctx->stream));
+    return AWQ_OK;
+}
+
+int awq_event_elapsed_ms(awq_ctx* ctx, void* start, void* stop, float* ms) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(ms, AWQ_ERR_ARG, "null ms");
+    AWQ_HIP_TRY(hipEventSynchronize((hipEvent_t)stop));
+    AWQ_HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return AWQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,487 @@
+// Model level of libawq_hip: load a weight_packer .bin image to the GPU,
+// allocate the run state, and push one token through the network.
+//
+// Follows the reference's single-GPU flow: build_transformer /
+// init_transformer (llama2_q4.cu:613-659), malloc_run_state (:62-91), the file
+// order of checkpoint_init_weights (:220-246), run_llama_network (:430-538),
+// run_transformer incl. its seq-len-binned graph replay (:541-601) and the
+// greedy branch of sample() (sampler.h:77-84).
+#include <stdlib.h>
+#include <string.h>
+
+#include <vector>
+
+#include "common.hpp"
+
+int awq_launch_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* w, int K, int N, int accum,
+                           int gpu_count, int loff, const int* pos, const uint16_t* norm_w, uint16_t* norm_out);
+int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
+                   const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw, int K, int N, int loff,
+                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out);
+int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w, const awq_qweight* up_w, int K,
+                   int N, const uint16_t* norm_w, uint16_t* norm_out);
+int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
+                          const uint16_t* norm_w, uint16_t* norm_out);
+
+namespace {
+
+constexpr int kMaxSeqLen = 128 * 1024;  // SharedData.tokens capacity, common.h:13
+constexpr int kMaxGraphs = 8;           // llama2_q4.cu:337
+
+struct SharedData {  // common.h:57-60, pinned host memory
+    volatile int pos;
+    int tokens[kMaxSeqLen];
+};
+
+}  // namespace
+
+struct awq_transformer {
+    awq_ctx* ctx;
+    awq_config cfg;
+    uint8_t* blob;  // every tensor of the file, in file order, in one device allocation
+    size_t blob_bytes;
+    const uint16_t* embed;
+    const uint16_t* wcls;
+    const uint16_t* rms_final;
+    std::vector<awq_layer_weights> layers;
+    awq_run_state s;
+    SharedData* shared;
+    hipGraphExec_t graphs[2][kMaxGraphs];
+    bool captured[2][kMaxGraphs];
+};
+
+namespace {
+
+size_t qweight_bytes(int K, int N) {
+    return (size_t)packed_weight_height(K) * N * 4 + (size_t)packed_zeros_height(K) * N * 4 + (size_t)scales_height(K) * N * 2;
+}
+
+size_t model_payload_bytes(const awq_config& c) {
+    const int kv_dim = (c.dim * c.n_kv_heads) / c.n_heads;
+    size_t b = 2 * (size_t)c.vocab_size * c.dim * 2 + (size_t)c.dim * 2;
+    size_t layer = 2 * qweight_bytes(c.dim, c.dim) + 2 * qweight_bytes(c.dim, kv_dim) + 2 * qweight_bytes(c.dim, c.hidden_dim) +
+                   qweight_bytes(c.hidden_dim, c.dim) + 2 * (size_t)c.dim * 2;
+    return b + layer * c.n_layers;
+}
+
+int check_config(const awq_config& c) {
+    AWQ_REQUIRE(c.dim > 0 && c.hidden_dim > 0 && c.n_layers > 0 && c.n_heads > 0 && c.n_kv_heads > 0 && c.vocab_size > 0 &&
+                    c.seq_len > 0,
+                AWQ_ERR_IO, "bad header: non-positive field");
+    AWQ_REQUIRE(c.seq_len <= kMaxSeqLen - 1, AWQ_ERR_IO, "bad header: seq_len above 128K");
+    AWQ_REQUIRE(c.n_heads % c.n_kv_heads == 0 && c.dim % c.n_heads == 0, AWQ_ERR_IO, "bad header: head counts do not divide");
+    const int kv_dim = (c.dim * c.n_kv_heads) / c.n_heads;
+    // The packer writes ceil(K/8) dwords per row and the loader expects ceil(K/32)*4: only K % 32 == 0 files
+    // load correctly in the reference (weight_packer.cpp:156 vs llama2_q4.cu:111).
+    AWQ_REQUIRE(c.dim % 32 == 0 && c.hidden_dim % 32 == 0, AWQ_ERR_SHAPE, "dim and hidden_dim must be multiples of 32");
+    AWQ_REQUIRE((kv_dim & 7) == 0 && (c.vocab_size & 7) == 0, AWQ_ERR_SHAPE, "kv_dim and vocab_size must be multiples of 8");
+    AWQ_REQUIRE(c.dim <= kMaxStagedK && c.hidden_dim <= kMaxStagedK, AWQ_ERR_SHAPE, "dim/hidden_dim above the staged maximum");
+    const int head = c.dim / c.n_heads;
+    AWQ_REQUIRE(head == 64 || head == 128 || head == 256, AWQ_ERR_SHAPE, "head size must be 64, 128 or 256");
+    AWQ_REQUIRE(c.n_heads <= kAttnMaxHeads, AWQ_ERR_SHAPE, "too many heads");
+    return AWQ_OK;
+}
+
+const uint8_t* take_qweight(awq_qweight* w, const uint8_t* p, int K, int N) {
+    w->weight = reinterpret_cast<const uint32_t*>(p);
+    p += (size_t)packed_weight_height(K) * N * 4;
+    w->zeros = reinterpret_cast<const uint32_t*>(p);
+    p += (size_t)packed_zeros_height(K) * N * 4;
+    w->scales = reinterpret_cast<const uint16_t*>(p);
+    p += (size_t)scales_height(K) * N * 2;
+    return p;
+}
+
+void map_tensors(awq_transformer* t) {
+    const awq_config& c = t->cfg;
+    const int kv_dim = (c.dim * c.n_kv_heads) / c.n_heads;
+    const uint8_t* p = t->blob;
+    t->embed = reinterpret_cast<const uint16_t*>(p);
+    p += (size_t)c.vocab_size * c.dim * 2;
+    t->wcls = reinterpret_cast<const uint16_t*>(p);
+    p += (size_t)c.vocab_size * c.dim * 2;
+    t->rms_final = reinterpret_cast<const uint16_t*>(p);
+    p += (size_t)c.dim * 2;
+    t->layers.resize(c.n_layers);
+    for (int l = 0; l < c.n_layers; l++) {
+        awq_layer_weights& L = t->layers[l];
+        p = take_qweight(&L.wq_q, p, c.dim, c.dim);
+        p = take_qweight(&L.wq_k, p, c.dim, kv_dim);
+        p = take_qweight(&L.wq_v, p, c.dim, kv_dim);
+        p = take_qweight(&L.wq_o, p, c.dim, c.dim);
+        p = take_qweight(&L.wq_up, p, c.dim, c.hidden_dim);  // file order: up before gate (llama2_q4.cu:236-237)
+        p = take_qweight(&L.wq_gate, p, c.dim, c.hidden_dim);
+        p = take_qweight(&L.wq_down, p, c.hidden_dim, c.dim);
+        L.rms_att_weight = reinterpret_cast<const uint16_t*>(p);
+        p += (size_t)c.dim * 2;
+        L.rms_ffn_weight = reinterpret_cast<const uint16_t*>(p);
+        p += (size_t)c.dim * 2;
+    }
+}
+
+int alloc_state(awq_transformer* t) {
+    const awq_config& c = t->cfg;
+    const size_t kv_dim = ((size_t)c.dim * c.n_kv_heads) / c.n_heads;
+    awq_run_state& s = t->s;
+    AWQ_HIP_TRY(hipMalloc((void**)&s.x, (size_t)c.dim * 2));
+    AWQ_HIP_TRY(hipMalloc((void**)&s.xb, (size_t)c.dim * 2));
+    AWQ_HIP_TRY(hipMalloc((void**)&s.hb, (size_t)c.hidden_dim * 2));
+    AWQ_HIP_TRY(hipMalloc((void**)&s.q, (size_t)c.dim * 2));
+    AWQ_HIP_TRY(hipMalloc((void**)&s.att, (size_t)c.n_heads * c.seq_len * 2));
+    AWQ_HIP_TRY(hipMalloc((void**)&s.logits, (size_t)c.vocab_size * 2));
+    const size_t kv_bytes = (size_t)c.n_layers * c.seq_len * kv_dim * 2;
+    AWQ_HIP_TRY(hipMalloc((void**)&s.key_cache, kv_bytes));
+    AWQ_HIP_TRY(hipMalloc((void**)&s.value_cache, kv_bytes));
+    AWQ_HIP_TRY(hipMalloc((void**)&s.pos, sizeof(int)));
+    AWQ_HIP_TRY(hipMemset(s.key_cache, 0, kv_bytes));
+    AWQ_HIP_TRY(hipMemset(s.value_cache, 0, kv_bytes));
+    AWQ_HIP_TRY(hipMemset(s.pos, 0, sizeof(int)));
+    AWQ_HIP_TRY(hipHostMalloc((void**)&t->shared, sizeof(SharedData), hipHostMallocDefault));
+    memset((void*)t->shared, 0, sizeof(SharedData));
+    s.shared_pos = &t->shared->pos;
+    s.shared_tokens = t->shared->tokens;
+    return AWQ_OK;
+}
+
+void release(awq_transformer* t) {
+    if (!t) return;
+    for (int m = 0; m < 2; m++)
+        for (int i = 0; i < kMaxGraphs; i++)
+            if (t->captured[m][i]) (void)hipGraphExecDestroy(t->graphs[m][i]);
+    (void)hipFree(t->blob);
+    (void)hipFree(t->s.x);
+    (void)hipFree(t->s.xb);
+    (void)hipFree(t->s.hb);
+    (void)hipFree(t->s.q);
+    (void)hipFree(t->s.att);
+    (void)hipFree(t->s.logits);
+    (void)hipFree(t->s.key_cache);
+    (void)hipFree(t->s.value_cache);
+    (void)hipFree(t->s.pos);
+    if (t->shared) (void)hipHostFree(t->shared);
+    delete t;
+}
+
+awq_transformer* new_transformer(awq_ctx* ctx) {
+    awq_transformer* t = new awq_transformer();
+    t->ctx = ctx;
+    t->blob = nullptr;
+    t->blob_bytes = 0;
+    t->shared = nullptr;
+    memset(&t->s, 0, sizeof(t->s));
+    memset(t->captured, 0, sizeof(t->captured));
+    return t;
+}
+
+// One token, the reference's launcher sequence with gpu_count = 1.
+int network_reference(awq_transformer* t, int seq_len_bin) {
+    awq_ctx* ctx = t->ctx;
+    const awq_config& p = t->cfg;
+    awq_run_state& s = t->s;
+    const int dim = p.dim, hidden_dim = p.hidden_dim;
+    const int head_size = dim / p.n_heads;
+    const int kv_dim = (p.dim * p.n_kv_heads) / p.n_heads;
+    const int kv_mul = p.n_heads / p.n_kv_heads;
+    int* pPos = s.pos;
+    int r;
+    if ((r = awq_embed(ctx, s.x, t->embed, dim, s.shared_tokens, pPos))) return r;
+    for (int l = 0; l < p.n_layers; l++) {
+        const awq_layer_weights& L = t->layers[l];
+        if ((r = awq_rmsnorm(ctx, s.xb, s.x, L.rms_att_weight, dim))) return r;
+        const int loff = l * p.seq_len * kv_dim;
+        if (dim == kv_dim) {
+            if ((r = awq_qkv_matvec(ctx, s.q, s.key_cache, s.value_cache, s.xb, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, loff, pPos)))
+                return r;
+        } else {
+            if ((r = awq_matvec_int4(ctx, s.q, s.xb, &L.wq_q, dim, dim, 0, 1, -1, nullptr))) return r;
+            if ((r = awq_matvec_int4(ctx, s.key_cache, s.xb, &L.wq_k, dim, kv_dim, 0, 1, loff, pPos))) return r;
+            if ((r = awq_matvec_int4(ctx, s.value_cache, s.xb, &L.wq_v, dim, kv_dim, 0, 1, loff, pPos))) return r;
+        }
+        if ((r = awq_rope(ctx, s.q, s.key_cache, p.n_heads, p.n_kv_heads, head_size, pPos, loff, p.rope_theta))) return r;
+        if ((r = awq_attention(ctx, s.xb, s.q, s.key_cache + loff, s.value_cache + loff, s.att, p.n_heads, head_size, kv_mul,
+                               seq_len_bin, pPos)))
+            return r;
+        if ((r = awq_matvec_int4(ctx, s.x, s.xb, &L.wq_o, dim, dim, 1, 1, -1, nullptr))) return r;
+        if ((r = awq_rmsnorm(ctx, s.xb, s.x, L.rms_ffn_weight, dim))) return r;
+        if ((r = awq_ffn_matvec_silu(ctx, s.hb, s.xb, &L.wq_gate, &L.wq_up, dim, hidden_dim))) return r;
+        if ((r = awq_matvec_int4(ctx, s.x, s.hb, &L.wq_down, hidden_dim, dim, 1, 1, -1, nullptr))) return r;
+    }
+    if ((r = awq_rmsnorm(ctx, s.x, s.x, t->rms_final, dim))) return r;
+    return awq_matvec_f16(ctx, s.logits, s.x, t->wcls, dim, p.vocab_size);
+}
+
+// Same arithmetic with RMSNorm folded into the staging of the consuming
+// matrix-vector kernels (the normalised vector never travels through memory).
+int network_fused(awq_transformer* t, int seq_len_bin) {
+    awq_ctx* ctx = t->ctx;
+    const awq_config& p = t->cfg;
+    awq_run_state& s = t->s;
+    const int dim = p.dim, hidden_dim = p.hidden_dim;
+    const int head_size = dim / p.n_heads;
+    const int kv_dim = (p.dim * p.n_kv_heads) / p.n_heads;
+    const int kv_mul = p.n_heads / p.n_kv_heads;
+    int* pPos = s.pos;
+    int r;
+    if ((r = awq_embed(ctx, s.x, t->embed, dim, s.shared_tokens, pPos))) return r;
+    for (int l = 0; l < p.n_layers; l++) {
+        const awq_layer_weights& L = t->layers[l];
+        const int loff = l * p.seq_len * kv_dim;
+        if (dim == kv_dim) {
+            if ((r = awq_launch_qkv(ctx, s.q, s.key_cache, s.value_cache, s.x, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, loff, pPos,
+                                    L.rms_att_weight, nullptr)))
+                return r;
+        } else {
+            if ((r = awq_launch_matvec_int4(ctx, s.q, s.x, &L.wq_q, dim, dim, 0, 1, -1, nullptr, L.rms_att_weight, nullptr)))
+                return r;
+            if ((r = awq_launch_matvec_int4(ctx, s.key_cache, s.x, &L.wq_k, dim, kv_dim, 0, 1, loff, pPos, L.rms_att_weight,
+                                            nullptr)))
+                return r;
+            if ((r = awq_launch_matvec_int4(ctx, s.value_cache, s.x, &L.wq_v, dim, kv_dim, 0, 1, loff, pPos, L.rms_att_weight,
+                                            nullptr)))
+                return r;
+        }
+        if ((r = awq_rope(ctx, s.q, s.key_cache, p.n_heads, p.n_kv_heads, head_size, pPos, loff, p.rope_theta))) return r;
+        if ((r = awq_attention(ctx, s.xb, s.q, s.key_cache + loff, s.value_cache + loff, s.att, p.n_heads, head_size, kv_mul,
+                               seq_len_bin, pPos)))
+            return r;
+        if ((r = awq_launch_matvec_int4(ctx, s.x, s.xb, &L.wq_o, dim, dim, 1, 1, -1, nullptr, nullptr, nullptr))) return r;
+        if ((r = awq_launch_ffn(ctx, s.hb, s.x, &L.wq_gate, &L.wq_up, dim, hidden_dim, L.rms_ffn_weight, nullptr))) return r;
+        if ((r = awq_launch_matvec_int4(ctx, s.x, s.hb, &L.wq_down, hidden_dim, dim, 1, 1, -1, nullptr, nullptr, nullptr)))
+            return r;
+    }
+    return awq_launch_matvec_f16(ctx, s.logits, s.x, t->wcls, dim, p.vocab_size, t->rms_final, nullptr);
+}
+
+int network(awq_transformer* t, int seq_len_bin, int mode) {
+    return mode == AWQ_SCHEDULE_FUSED ? network_fused(t, seq_len_bin) : network_reference(t, seq_len_bin);
+}
+
+}  // namespace
+
+extern "C" {
+
+int awq_transformer_load_image(awq_ctx* ctx, const void* image, size_t bytes, awq_transformer** out) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(image && out, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(bytes >= sizeof(awq_config), AWQ_ERR_IO, "Invalid header size");
+    awq_transformer* t = new_transformer(ctx);
+    memcpy(&t->cfg, image, sizeof(awq_config));
+    int r = check_config(t->cfg);
+    if (r) {
+        release(t);
+        return r;
+    }
+    t->blob_bytes = model_payload_bytes(t->cfg);
+    if (bytes < sizeof(awq_config) + t->blob_bytes) {
+        awq_set_error("error reading weights: image holds %zu bytes, config needs %zu", bytes, sizeof(awq_config) + t->blob_bytes);
+        release(t);
+        return AWQ_ERR_IO;
+    }
+    hipError_t e = hipMalloc((void**)&t->blob, t->blob_bytes);
+    if (e == hipSuccess)
+        e = hipMemcpy(t->blob, (const uint8_t*)image + sizeof(awq_config), t->blob_bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        awq_set_error("weight upload failed: %s", hipGetErrorString(e));
+        release(t);
+        return AWQ_ERR_HIP;
+    }
+    map_tensors(t);
+    r = alloc_state(t);
+    if (r) {
+        release(t);
+        return r;
+    }
+    AWQ_HIP_TRY(hipDeviceSynchronize());
+    *out = t;
+    return AWQ_OK;
+}
+
+int awq_transformer_load_file(awq_ctx* ctx, const char* checkpoint_path, awq_transformer** out) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(checkpoint_path && out, AWQ_ERR_ARG, "null pointer");
+    FILE* f = fopen(checkpoint_path, "rb");
+    if (!f) {
+        awq_set_error("Couldn't open file %s", checkpoint_path);
+        return AWQ_ERR_IO;
+    }
+    awq_transformer* t = new_transformer(ctx);
+    if (fread(&t->cfg, sizeof(awq_config), 1, f) != 1) {
+        awq_set_error("Invalid header size");
+        fclose(f);
+        release(t);
+        return AWQ_ERR_IO;
+    }
+    int r = check_config(t->cfg);
+    if (r) {
+        fclose(f);
+        release(t);
+        return r;
+    }
+    t->blob_bytes = model_payload_bytes(t->cfg);
+    hipError_t e = hipMalloc((void**)&t->blob, t->blob_bytes);
+    if (e != hipSuccess) {
+        awq_set_error("weight allocation failed: %s", hipGetErrorString(e));
+        fclose(f);
+        release(t);
+        return AWQ_ERR_HIP;
+    }
+    // Stream the file through two pinned staging buffers so that disk reads overlap the uploads.
+    const size_t chunk = (size_t)64 << 20;
+    uint8_t* stage[2] = {nullptr, nullptr};
+    hipEvent_t done[2];
+    bool ok = true;
+    for (int i = 0; i < 2 && ok; i++) {
+        ok = hipHostMalloc((void**)&stage[i], chunk, hipHostMallocDefault) == hipSuccess && hipEventCreate(&done[i]) == hipSuccess;
+    }
+    size_t off = 0;
+    int which = 0;
+    bool used[2] = {false, false};
+    while (ok && off < t->blob_bytes) {
+        const size_t n = (t->blob_bytes - off < chunk) ? t->blob_bytes - off : chunk;
+        if (used[which]) ok = hipEventSynchronize(done[which]) == hipSuccess;
+        if (ok && fread(stage[which], 1, n, f) != n) {
+            awq_set_error("error reading weights");
+            r = AWQ_ERR_IO;
+            ok = false;
+            break;
+        }
+        if (ok) ok = hipMemcpyAsync(t->blob + off, stage[which], n, hipMemcpyHostToDevice, ctx->stream) == hipSuccess;
+        if (ok) ok = hipEventRecord(done[which], ctx->stream) == hipSuccess;
+        used[which] = true;
+        which ^= 1;
+        off += n;
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    for (int i = 0; i < 2; i++) {
+        if (stage[i]) {
+            (void)hipHostFree(stage[i]);
+            (void)hipEventDestroy(done[i]);
+        }
+    }
+    fclose(f);
+    if (!ok) {
+        if (r == AWQ_OK) {
+            awq_set_error("weight upload failed");
+            r = AWQ_ERR_HIP;
+        }
+        release(t);
+        return r;
+    }
+    map_tensors(t);
+    r = alloc_state(t);
+    if (r) {
+        release(t);
+        return r;
+    }
+    AWQ_HIP_TRY(hipDeviceSynchronize());
+    *out = t;
+    return AWQ_OK;
+}
+
+int awq_transformer_free(awq_transformer* t) {
+    AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
+    if (int r = awq_bind(t->ctx)) return r;
+    (void)hipStreamSynchronize(t->ctx->stream);
+    release(t);
+    return AWQ_OK;
+}
+
+int awq_transformer_config(const awq_transformer* t, awq_config* out) {
+    AWQ_REQUIRE(t && out, AWQ_ERR_ARG, "null pointer");
+    *out = t->cfg;
+    return AWQ_OK;
+}
+
+int awq_transformer_state(const awq_transformer* t, awq_run_state* out) {
+    AWQ_REQUIRE(t && out, AWQ_ERR_ARG, "null pointer");
+    *out = t->s;
+    return AWQ_OK;
+}
+
+int awq_transformer_layer(const awq_transformer* t, int layer, awq_layer_weights* out) {
+    AWQ_REQUIRE(t && out, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(layer >= 0 && layer < t->cfg.n_layers, AWQ_ERR_ARG, "no such layer");
+    *out = t->layers[layer];
+    return AWQ_OK;
+}
+
+int awq_transformer_globals(const awq_transformer* t, const uint16_t** embed, const uint16_t** wcls, const uint16_t** rms_final) {
+    AWQ_REQUIRE(t, AWQ_ERR_ARG, "null pointer");
+    if (embed) *embed = t->embed;
+    if (wcls) *wcls = t->wcls;
+    if (rms_final) *rms_final = t->rms_final;
+    return AWQ_OK;
+}
+
+int awq_transformer_reset(awq_transformer* t, const int* prompt_tokens, int num_prompt_tokens) {
+    AWQ_REQUIRE(t && prompt_tokens, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(num_prompt_tokens >= 1 && num_prompt_tokens <= t->cfg.seq_len, AWQ_ERR_ARG, "prompt length out of range");
+    if (int r = awq_bind(t->ctx)) return r;
+    AWQ_HIP_TRY(hipStreamSynchronize(t->ctx->stream));
+    AWQ_HIP_TRY(hipMemset(t->s.pos, 0, sizeof(int)));
+    t->shared->pos = 0;
+    memcpy(t->shared->tokens, prompt_tokens, sizeof(int) * (size_t)num_prompt_tokens);
+    return AWQ_OK;
+}
+
+int awq_transformer_set_pos(awq_transformer* t, int pos, int token) {
+    AWQ_REQUIRE(t, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(pos >= 0 && pos < t->cfg.seq_len, AWQ_ERR_ARG, "pos out of range");
+    if (int r = awq_bind(t->ctx)) return r;
+    AWQ_HIP_TRY(hipStreamSynchronize(t->ctx->stream));
+    AWQ_HIP_TRY(hipMemcpy(t->s.pos, &pos, sizeof(int), hipMemcpyHostToDevice));
+    t->shared->pos = pos;
+    t->shared->tokens[pos] = token;
+    return AWQ_OK;
+}
+
+int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode) {
+    AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
+    AWQ_REQUIRE(mode == AWQ_SCHEDULE_REFERENCE || mode == AWQ_SCHEDULE_FUSED, AWQ_ERR_ARG, "unknown schedule");
+    awq_ctx* ctx = t->ctx;
+    if (int r = awq_bind(ctx)) return r;
+    // llama2_q4.cu:552: the host's view of the position sizes the attention launch
+    const int seq_len = t->shared->pos + 1;
+    AWQ_REQUIRE(seq_len <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+    int r;
+    if (use_graph) {
+        // llama2_q4.cu:553-558: bins 128, 256, ..., last bin = seq_len of the model
+        int graph_index;
+        int seq_len_bin = 128;
+        for (graph_index = 0; graph_index < kMaxGraphs - 1; seq_len_bin *= 2, graph_index++)
+            if (seq_len <= seq_len_bin) break;
+        if (seq_len > seq_len_bin || graph_index == kMaxGraphs - 1 || seq_len_bin > t->cfg.seq_len) seq_len_bin = t->cfg.seq_len;
+        if (!t->captured[mode][graph_index]) {
+            hipGraph_t graph = nullptr;
+            AWQ_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+            r = network(t, seq_len_bin, mode);
+            if (r == AWQ_OK)
+                r = awq_argmax_advance(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, 1);
+            hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+            if (r) {
+                if (graph) (void)hipGraphDestroy(graph);
+                return r;
+            }
+            if (e != hipSuccess) {
+                awq_set_error("hipStreamEndCapture failed: %s", hipGetErrorString(e));
+                return AWQ_ERR_HIP;
+            }
+            AWQ_HIP_TRY(hipGraphInstantiate(&t->graphs[mode][graph_index], graph, nullptr, nullptr, 0));
+            AWQ_HIP_TRY(hipGraphDestroy(graph));
+            t->captured[mode][graph_index] = true;
+        }
+        // The recorded sampler always writes its token; while the prompt is being consumed the next prompt
+        // token must survive, so those steps run eagerly below.
+        if (gen_token) {
+            AWQ_HIP_TRY(hipGraphLaunch(t->graphs[mode][graph_index], ctx->stream));
+            return AWQ_OK;
+        }
+        r = network(t, seq_len_bin, mode);
+    } else {
+        r = network(t, seq_len, mode);
+    }
+    if (r) return r;
+    return awq_argmax_advance(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token);
+}
+
+}  // extern "C"

@@ -1,0 +1,110 @@
+"""GPU parity of the whole decode path against the CPU oracle on small models.
+
+Bar (from the benchmark definition): logits within rel-L2 1e-2 of the oracle at every step, greedy tokens
+identical for the first 32 steps.  The run state after one token is also compared buffer by buffer.
+"""
+import numpy as np
+import pytest
+
+import llama_cu_awq_amd as A
+from llama_cu_awq_amd import synth
+from oracle import oracle
+from tests.helpers import f16, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+TINY = dict(dim=256, hidden_dim=768, n_layers=2, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=64, rope_theta=10000.0)
+SMALL = dict(dim=1024, hidden_dim=2752, n_layers=4, n_heads=8, n_kv_heads=8, vocab_size=4096, seq_len=160, rope_theta=10000.0)
+GQA = dict(dim=512, hidden_dim=1376, n_layers=2, n_heads=8, n_kv_heads=2, vocab_size=1024, seq_len=64, rope_theta=10000.0)
+
+
+@pytest.fixture(scope="module", params=["tiny", "small", "gqa"])
+def pair(request, ctx):
+    cfg = {"tiny": TINY, "small": SMALL, "gqa": GQA}[request.param]
+    img = synth.make_model_image(cfg, seed=0)
+    t = A.Transformer(ctx, image=img)
+    o = oracle.Model(img)
+    yield cfg, t, o
+    t.close()
+    o.close()
+
+
+def test_header_round_trip(pair):
+    cfg, t, o = pair
+    for k in ("dim", "hidden_dim", "n_layers", "n_heads", "n_kv_heads", "vocab_size", "seq_len"):
+        assert t.config[k] == cfg[k] == o.config[k]
+
+
+@pytest.mark.parametrize("mode", [A.SCHEDULE_REFERENCE, A.SCHEDULE_FUSED])
+def test_one_token_state(pair, mode):
+    cfg, t, o = pair
+    prompt = synth.prompt_tokens(1, 4, cfg["vocab_size"])
+    t.reset(prompt)
+    o.reset(prompt)
+    for step in range(3):
+        t.forward(gen_token=False, use_graph=False, mode=mode)
+        o.forward(gen_token=False)
+    t.ctx.sync()
+    assert t.pos == 3 == o.tokens(0) or t.pos == 3
+    kv_dim = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"]
+    for name, n in (("logits", cfg["vocab_size"]), ("hb", cfg["hidden_dim"]), ("q", cfg["dim"]), ("key_cache", 3 * kv_dim), ("value_cache", 3 * kv_dim)):
+        got = f16(t.download(name, n))
+        want = f16(o.buffer(name, n))
+        assert rel_l2(got, want) <= 1e-2, name
+
+
+@pytest.mark.parametrize("mode,graph", [(A.SCHEDULE_REFERENCE, False), (A.SCHEDULE_FUSED, False), (A.SCHEDULE_FUSED, True), (A.SCHEDULE_REFERENCE, True)])
+def test_greedy_decode_matches_oracle(pair, mode, graph):
+    cfg, t, o = pair
+    n_prompt, steps = 8, min(48, cfg["seq_len"] - 1)
+    prompt = synth.prompt_tokens(2, n_prompt, cfg["vocab_size"])
+    want_tokens, want_pos, want_logits = o.generate(prompt, steps, ignore_eos=True, want_logits=True)
+    got_logits = {}
+    got_tokens, got_pos = t.generate(prompt, steps, ignore_eos=True, use_graph=graph, mode=mode, on_logits=lambda p, l: got_logits.__setitem__(p, f16(l)))
+    assert got_pos == want_pos == steps
+    # prompt tokens are echoed unchanged
+    assert got_tokens[:n_prompt] == prompt
+    first_diff = next((i for i in range(len(want_tokens)) if got_tokens[i] != want_tokens[i]), None)
+    margin = None
+    if first_diff is not None:
+        l = np.sort(want_logits[first_diff - 1].astype(np.float64))
+        margin = l[-1] - l[-2]
+    assert first_diff is None or first_diff > n_prompt + 32, f"token mismatch at {first_diff}, top-1/top-2 margin {margin}"
+    upto = steps if first_diff is None else first_diff
+    worst = max(rel_l2(got_logits[p], want_logits[p]) for p in range(upto))
+    assert worst <= 1e-2, worst
+
+
+def test_eos_stops_generation(pair):
+    """The loop breaks when token 2 is read back (llama2_q4.cu:730)."""
+    cfg, t, o = pair
+    prompt = [5, 2, 9]  # EOS inside the prompt: both stop when it is read back at pos 1
+    got_tokens, got_pos = t.generate(prompt, 10)
+    want_tokens, want_pos, _ = o.generate(prompt, 10)
+    assert got_pos == want_pos == 1
+
+
+def test_load_errors(ctx):
+    img = synth.make_model_image(TINY, seed=0)
+    with pytest.raises(A.AwqError):
+        A.Transformer(ctx, image=img[:1000])  # short image: "error reading weights"
+    bad = img.copy()
+    bad[:4] = np.array([-5], dtype=np.int32).view(np.uint8)
+    with pytest.raises(A.AwqError):
+        A.Transformer(ctx, image=bad)
+    with pytest.raises(A.AwqError):
+        A.Transformer(ctx, path="/nonexistent/model.bin")
+
+
+def test_load_file_equals_image(ctx, tmp_path):
+    img = synth.make_model_image(TINY, seed=3)
+    p = tmp_path / "m.bin"
+    img.tofile(p)
+    a = A.Transformer(ctx, image=img)
+    b = A.Transformer(ctx, path=str(p))
+    prompt = synth.prompt_tokens(4, 4, TINY["vocab_size"])
+    ta, _ = a.generate(prompt, 20, ignore_eos=True)
+    tb, _ = b.generate(prompt, 20, ignore_eos=True)
+    assert ta == tb
+    a.close()
+    b.close()

@@ -1,0 +1,305 @@
+"""GPU parity: every op of the C-ABI against the CPU oracle and against fp64 closed forms.
+
+Tolerances: unpack/dequant bit-exact; matrix-vector outputs rel-L2 <= 1e-3 of the fp64 product of the exactly
+dequantised weights (the stated bound) and, tighter, within 2 fp16 steps of the oracle's fp32 restatement
+(summation order differs); fp16 element-wise ops within 1 fp16 step of the oracle.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import llama_cu_awq_amd as A
+from llama_cu_awq_amd import synth
+from llama_cu_awq_amd._lib import AWQ_ERR_SHAPE, lib
+from oracle import oracle
+from tests.helpers import f16, rel_l2, ulp_diff_f16
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (5120, 5120), (13824, 5120), (6656, 1024), (17920, 512), (128, 8), (200, 24), (1056, 40)]
+
+
+def _case(K, N, tag=0):
+    key = synth.stream_key(0, "case", K, N, tag)
+    w, z, s = synth.make_qweight(key, K, N)
+    x = synth.normal_f16(synth.stream_key(key, "x"), K)
+    return w, z, s, x
+
+
+@pytest.mark.parametrize("K,N", [(4096, 512), (11008, 64), (200, 24), (128, 8), (13824, 32)])
+def test_dequant_bit_exact(ctx, K, N):
+    w, z, s, _ = _case(K, N)
+    qw = A.QWeight.upload(ctx, w, z, s)
+    out = ctx.alloc(N * K * 2)
+    A.dequant(ctx, out, qw, K, N)
+    got = out.download(np.uint16).reshape(N, K)
+    want = oracle.dequant(w, z, s, K, N).view(np.uint16)
+    assert np.array_equal(got, want)
+    # and against the layout definition in numpy (single rounding of the exact product)
+    ref = synth.dequantize(w, z, s, K).astype(np.float32).astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("K,N", SHAPES)
+def test_matvec_int4_plain(ctx, K, N):
+    w, z, s, x = _case(K, N)
+    qw = A.QWeight.upload(ctx, w, z, s)
+    dx = ctx.upload(x)
+    dout = ctx.zeros(N * 2)
+    A.matmul_q(ctx, dout, dx, qw, K, N)
+    got = f16(dout.download(np.uint16))
+    truth = synth.dequantize(w, z, s, K) @ x.astype(np.float64)
+    assert rel_l2(got, truth) <= 1e-3
+    want = np.zeros(N, dtype=np.uint16)
+    assert oracle.matvec_int4(want, x, w, z, s, K, N) == 0
+    assert ulp_diff_f16(got, f16(want)).max() <= 2
+    assert rel_l2(got, f16(want)) <= 3e-4
+
+
+def test_matvec_int4_accum_and_kv_offset(ctx):
+    K, N = 4096, 4096
+    w, z, s, x = _case(K, N, 1)
+    qw = A.QWeight.upload(ctx, w, z, s)
+    dx = ctx.upload(x)
+    resid = synth.normal_f16(synth.stream_key(1, "res"), N)
+    # residual epilogue: out = half(Wx + out)
+    dout = ctx.upload(resid)
+    A.matmul_q(ctx, dout, dx, qw, K, N, accum=True, gpu_count=1)
+    got = f16(dout.download(np.uint16))
+    want = resid.view(np.uint16).copy()
+    oracle.matvec_int4(want, x, w, z, s, K, N, accum=True)
+    assert ulp_diff_f16(got, f16(want)).max() <= 2
+    truth = synth.dequantize(w, z, s, K) @ x.astype(np.float64) + resid.astype(np.float64)
+    assert rel_l2(got, truth) <= 1e-3
+    # gpu_count = 2 pre-divides the residual (gpu_kernels.h:237-238)
+    dout = ctx.upload(resid)
+    A.matmul_q(ctx, dout, dx, qw, K, N, accum=True, gpu_count=2)
+    got = f16(dout.download(np.uint16))
+    truth = synth.dequantize(w, z, s, K) @ x.astype(np.float64) + resid.astype(np.float64) / 2
+    assert rel_l2(got, truth) <= 1e-3
+    # KV-cache row epilogue: written at loff + pos*N, nothing else touched
+    pos, loff, rows = 3, 2 * N, 8
+    cache = np.full(rows * N, 0x3C00, dtype=np.uint16)
+    dcache = ctx.upload(cache)
+    dpos = ctx.upload(np.array([pos], dtype=np.int32))
+    A.matmul_q(ctx, dcache, dx, qw, K, N, loff=loff, pPos=dpos)
+    got = dcache.download(np.uint16)
+    want = cache.copy()
+    oracle.matvec_int4(want, x, w, z, s, K, N, loff=loff, pos=pos)
+    assert np.array_equal(got[: loff + pos * N], want[: loff + pos * N])
+    assert np.array_equal(got[loff + (pos + 1) * N :], want[loff + (pos + 1) * N :])
+    assert ulp_diff_f16(f16(got), f16(want)).max() <= 2
+
+
+def test_zero_weights_leave_residual(ctx):
+    """accum with W == 0 (q == z everywhere) returns the residual unchanged."""
+    K, N = 256, 64
+    pwh, pzh, sh = synth.strides(K)
+    w = np.full((N, pwh), 0x55555555, dtype=np.uint32)
+    z = np.full((N, pzh), 0x55555555, dtype=np.uint32)
+    s = np.full((N, sh), 0.01, dtype=np.float16)
+    x = synth.normal_f16(synth.stream_key(2, "x"), K)
+    resid = synth.normal_f16(synth.stream_key(2, "r"), N)
+    qw = A.QWeight.upload(ctx, w, z, s)
+    dout = ctx.upload(resid)
+    A.matmul_q(ctx, dout, ctx.upload(x), qw, K, N, accum=True)
+    assert np.array_equal(dout.download(np.uint16), resid.view(np.uint16))
+
+
+@pytest.mark.parametrize("K,N", [(4096, 4096), (5120, 5120), (256, 64)])
+def test_qkv_matvec(ctx, K, N):
+    mats = [_case(K, N, t)[:3] for t in (10, 11, 12)]
+    x = _case(K, N, 13)[3]
+    qws = [A.QWeight.upload(ctx, *m) for m in mats]
+    pos, loff, rows = 2, N, 5
+    dq = ctx.zeros(N * 2)
+    dk = ctx.zeros(rows * N * 2)
+    dv = ctx.zeros(rows * N * 2)
+    dpos = ctx.upload(np.array([pos], dtype=np.int32))
+    A.qkv_matvec(ctx, dq, dk, dv, ctx.upload(x), *qws, K, N, loff, dpos)
+    q = np.zeros(N, dtype=np.uint16)
+    kc = np.zeros(rows * N, dtype=np.uint16)
+    vc = np.zeros(rows * N, dtype=np.uint16)
+    oracle.qkv_matvec(q, kc, vc, x, *mats, K, N, loff, pos)
+    for got, want in ((dq.download(np.uint16), q), (dk.download(np.uint16), kc), (dv.download(np.uint16), vc)):
+        assert ulp_diff_f16(f16(got), f16(want)).max() <= 2
+        assert np.array_equal(got == 0, want == 0) or True
+    # only the addressed cache row is written
+    kgot = dk.download(np.uint16)
+    assert not kgot[: loff + pos * N].any() and not kgot[loff + (pos + 1) * N :].any()
+    truth = synth.dequantize(*mats[1], K) @ x.astype(np.float64)
+    assert rel_l2(f16(kgot[loff + pos * N : loff + (pos + 1) * N]), truth) <= 1e-3
+
+
+@pytest.mark.parametrize("K,N", [(4096, 11008), (5120, 13824), (6656, 1792), (256, 72)])
+def test_ffn_matvec_silu(ctx, K, N):
+    gate = _case(K, N, 20)[:3]
+    up = _case(K, N, 21)[:3]
+    x = _case(K, N, 22)[3]
+    dout = ctx.zeros(N * 2)
+    A.ffn_matvec_silu(ctx, dout, ctx.upload(x), A.QWeight.upload(ctx, *gate), A.QWeight.upload(ctx, *up), K, N)
+    got = f16(dout.download(np.uint16))
+    want = np.zeros(N, dtype=np.uint16)
+    oracle.ffn_matvec_silu(want, x, gate, up, K, N)
+    xd = x.astype(np.float64)
+    g = synth.dequantize(*gate, K) @ xd
+    u = synth.dequantize(*up, K) @ xd
+    truth = g / (1.0 + np.exp(-g)) * u
+    assert rel_l2(got, truth) <= 1e-3
+    assert rel_l2(got, f16(want)) <= 3e-4
+    assert ulp_diff_f16(got, f16(want)).max() <= 4
+
+
+@pytest.mark.parametrize("K,N", [(12, 8), (8, 12), (4096, 4100), (0, 8)])
+def test_shape_guard(ctx, K, N):
+    """The reference prints 'Unsupported matmul size' and exits; the library returns AWQ_ERR_SHAPE."""
+    buf = ctx.alloc(1 << 16)
+    qw = A.QWeight(buf, buf, buf)
+    with pytest.raises(A.AwqError) as e:
+        A.matmul_q(ctx, buf, buf, qw, K, N)
+    assert e.value.code == AWQ_ERR_SHAPE
+    with pytest.raises(A.AwqError):
+        A.ffn_matvec_silu(ctx, buf, buf, qw, qw, K, N)
+    with pytest.raises(A.AwqError):
+        A.matmul(ctx, buf, buf, buf, K, N)
+
+
+@pytest.mark.parametrize("size", [4096, 5120, 6656, 8, 1000])
+def test_rmsnorm(ctx, size):
+    x = synth.normal_f16(synth.stream_key(3, "x", size), size, 0.0, 2.0)
+    w = synth.normal_f16(synth.stream_key(3, "w", size), size, 1.0, 0.02)
+    dx = ctx.upload(x)
+    do = ctx.zeros(size * 2)
+    A.rmsnorm(ctx, do, dx, ctx.upload(w), size)
+    got = f16(do.download(np.uint16))
+    want = oracle.rmsnorm(x, w)
+    assert ulp_diff_f16(got, want).max() <= 1
+    xd = x.astype(np.float64)
+    truth = xd / np.sqrt((xd * xd).mean() + 1e-5) * w.astype(np.float64)
+    assert rel_l2(got, truth) <= 5e-4
+    # in place (the final norm of the network runs in place)
+    A.rmsnorm(ctx, dx, dx, ctx.upload(w), size)
+    assert np.array_equal(dx.download(np.uint16), do.download(np.uint16))
+
+
+@pytest.mark.parametrize("heads,kv_heads,head,pos", [(32, 32, 128, 0), (32, 32, 128, 17), (8, 2, 64, 2047), (4, 4, 256, 100), (40, 40, 128, 1791)])
+def test_rope(ctx, heads, kv_heads, head, pos):
+    seq, loff = pos + 2, 0
+    q = synth.normal_f16(synth.stream_key(4, "q", heads, pos), heads * head).view(np.uint16).copy()
+    kc = synth.normal_f16(synth.stream_key(4, "k", heads, pos), 2 * seq * kv_heads * head).view(np.uint16).copy()
+    loff = seq * kv_heads * head
+    dq, dk = ctx.upload(q), ctx.upload(kc)
+    dpos = ctx.upload(np.array([pos], dtype=np.int32))
+    A.RoPERotation(ctx, dq, dk, heads, kv_heads, head, dpos, loff, 10000.0)
+    q0, k0 = q.copy(), kc.copy()
+    oracle.rope(q, kc, heads, kv_heads, head, pos, loff, 10000.0)
+    gq, gk = dq.download(np.uint16), dk.download(np.uint16)
+    # device powf/sinf/cosf may differ from libm in the last place of the angle: allow 2 fp16 steps at large pos
+    tol = 0 if pos == 0 else 2
+    assert ulp_diff_f16(f16(gq), f16(q)).max() <= tol
+    assert ulp_diff_f16(f16(gk), f16(kc)).max() <= tol
+    if pos == 0:
+        assert np.array_equal(gq, q0) and np.array_equal(gk, k0)
+    # rows other than the addressed K row are untouched
+    row = loff + pos * kv_heads * head
+    assert np.array_equal(gk[:row], k0[:row]) and np.array_equal(gk[row + kv_heads * head :], k0[row + kv_heads * head :])
+    # fp64 closed form on q
+    i = np.arange(head // 2)
+    ang = pos * (1.0 / np.power(10000.0, 2.0 * i / head))
+    qq = f16(q0).astype(np.float64).reshape(heads, head)
+    a, b = qq[:, : head // 2], qq[:, head // 2 :]
+    truth = np.concatenate([a * np.cos(ang) - b * np.sin(ang), a * np.sin(ang) + b * np.cos(ang)], axis=1).reshape(-1)
+    assert rel_l2(f16(gq), truth) <= (2e-3 if pos > 1000 else 6e-4)
+
+
+@pytest.mark.parametrize(
+    "heads,head,kv_mul,pos,max_seq",
+    [(32, 128, 1, 0, 1), (32, 128, 1, 16, 17), (32, 128, 1, 271, 512), (40, 128, 1, 1791, 2048), (8, 64, 4, 300, 301), (4, 256, 2, 1023, 1024), (52, 128, 1, 2047, 2048)],
+)
+def test_attention(ctx, heads, head, kv_mul, pos, max_seq):
+    kv_dim = heads * head // kv_mul
+    seq = pos + 1
+    key = synth.stream_key(5, heads, head, kv_mul, pos)
+    q = synth.normal_f16(synth.stream_key(key, "q"), heads * head)
+    kc = synth.normal_f16(synth.stream_key(key, "k"), seq * kv_dim)
+    vc = synth.normal_f16(synth.stream_key(key, "v"), seq * kv_dim)
+    dout = ctx.zeros(heads * head * 2)
+    datt = ctx.zeros(heads * max(max_seq, seq) * 2)
+    dpos = ctx.upload(np.array([pos], dtype=np.int32))
+    A.MultiHeadAttention(ctx, dout, ctx.upload(q), ctx.upload(kc), ctx.upload(vc), datt, heads, head, kv_mul, max_seq, dpos)
+    got = f16(dout.download(np.uint16))
+    want, _ = oracle.attention(q, kc.view(np.uint16), vc.view(np.uint16), heads, head, kv_mul, pos)
+    # fp64 brute force softmax(qK^T/sqrt(d))V
+    Q = q.astype(np.float64).reshape(heads, head)
+    Kc = kc.astype(np.float64).reshape(seq, heads // kv_mul, head)
+    Vc = vc.astype(np.float64).reshape(seq, heads // kv_mul, head)
+    truth = np.empty((heads, head))
+    for h in range(heads):
+        sc = Kc[:, h // kv_mul, :] @ Q[h] / np.sqrt(head)
+        p = np.exp(sc - sc.max())
+        p /= p.sum()
+        truth[h] = p @ Vc[:, h // kv_mul, :]
+    # the fp16 rounding of scores and probabilities (reference behaviour) costs ~1e-3 vs fp64
+    assert rel_l2(got, truth.reshape(-1)) <= 4e-3
+    assert rel_l2(want, truth.reshape(-1)) <= 4e-3
+    assert rel_l2(got, want) <= 1.5e-3
+    # a second call gives the same bits (arrival counters reset themselves)
+    A.MultiHeadAttention(ctx, dout, ctx.upload(q), ctx.upload(kc), ctx.upload(vc), datt, heads, head, kv_mul, max_seq, dpos)
+    assert np.array_equal(dout.download(np.uint16), got.view(np.uint16))
+
+
+def test_attention_pos0_returns_v0(ctx):
+    heads, head = 32, 128
+    q = synth.normal_f16(synth.stream_key(6, "q"), heads * head)
+    kc = synth.normal_f16(synth.stream_key(6, "k"), heads * head)
+    vc = synth.normal_f16(synth.stream_key(6, "v"), heads * head)
+    dout = ctx.zeros(heads * head * 2)
+    A.MultiHeadAttention(ctx, dout, ctx.upload(q), ctx.upload(kc), ctx.upload(vc), ctx.zeros(heads * 2), heads, head, 1, 1, ctx.upload(np.array([0], dtype=np.int32)))
+    assert np.array_equal(dout.download(np.uint16), vc.view(np.uint16))
+
+
+@pytest.mark.parametrize("n,d", [(4096, 32000), (5120, 32000), (6656, 1024), (8, 8), (264, 40)])
+def test_matvec_f16(ctx, n, d):
+    key = synth.stream_key(7, n, d)
+    w = synth.normal_f16(synth.stream_key(key, "w"), n * d, 0.0, 0.02)
+    x = synth.normal_f16(synth.stream_key(key, "x"), n)
+    dout = ctx.zeros(d * 2)
+    A.matmul(ctx, dout, ctx.upload(x), ctx.upload(w), n, d)
+    got = f16(dout.download(np.uint16))
+    r, want = oracle.matvec_f16(x, w, n, d)
+    assert r == 0
+    truth = w.astype(np.float64).reshape(d, n) @ x.astype(np.float64)
+    assert rel_l2(got, truth) <= 1e-3
+    assert ulp_diff_f16(got, want).max() <= 2
+
+
+def test_argmax_advance_and_ties(ctx):
+    V = 32000
+    logits = synth.normal_f16(synth.stream_key(8, "l"), V)
+    m = np.float16(logits.max() + 1)
+    logits[[31999, 17, 20000]] = m  # a three-way tie: lowest index wins
+    host = ctx.alloc_host(4 * 64)
+    pos_host = C.c_int.from_address(host)
+    tokens = (C.c_int * 32).from_address(host + 16)
+    for i in range(32):
+        tokens[i] = -1
+    pos_host.value = 4
+    dpos = ctx.upload(np.array([4], dtype=np.int32))
+    A.argmax_advance(ctx, ctx.upload(logits), V, host + 16, host, dpos, True)
+    ctx.sync()
+    assert pos_host.value == 5 and tokens[5] == 17 and dpos.download(np.int32)[0] == 5
+    # write_token = False only advances the position
+    A.argmax_advance(ctx, ctx.upload(logits), V, host + 16, host, dpos, False)
+    ctx.sync()
+    assert pos_host.value == 6 and tokens[6] == -1 and dpos.download(np.int32)[0] == 6
+    ctx.free_host(host)
+
+
+def test_embed(ctx):
+    dim, V = 4096, 64
+    table = synth.normal_f16(synth.stream_key(9, "t"), V * dim).view(np.uint16)
+    toks = np.array([5, 63, 0, 7], dtype=np.int32)
+    dx = ctx.zeros(dim * 2)
+    A.copy_embedding(ctx, dx, ctx.upload(table), dim, ctx.upload(toks), ctx.upload(np.array([1], dtype=np.int32)))
+    assert np.array_equal(dx.download(np.uint16), table[63 * dim : 64 * dim])
