@@ -21,3 +21,18 @@ def ulp_diff_f16(a, b):
 
 def f16(bits):
     return np.asarray(bits, dtype=np.uint16).view(np.float16)
+
+
+def assert_close_f16(got, want, ulps=2, floor=2e-4):
+    """Each element within `ulps` fp16 steps of `want`, or within floor * rms(want) absolutely.
+
+    The absolute floor covers outputs that land near zero through cancellation, where an fp32
+    summation-order difference of ~1e-6 of the operand magnitude spans many fp16 steps.
+    """
+    got = np.asarray(got, dtype=np.float16)
+    want = np.asarray(want, dtype=np.float16)
+    d = ulp_diff_f16(got, want)
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    absd = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    bad = (d > ulps) & (absd > floor * rms)
+    assert not bad.any(), f"{int(bad.sum())} elements differ: worst {int(d[bad].max())} steps, abs {absd[bad].max():.3g} (rms {rms:.3g})"
