@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark: batch-1 greedy decode of a Llama-2-7B-shape AWQ int4-g128 model on one MI355X.
+
+A step is one token through the whole network (one pass of the hot path).  The default run consumes a 16-token
+random prompt as warm-up and times exactly 256 decode steps; weights are random (no checkpoints offline) with the
+real layout and distributions, resident in HBM before the timed region starts.
+
+Prints ONE JSON line: tokens/s (`value`), the roofline of the dominant kernel (the fused gate/up int4
+matrix-vector product) measured live with HIP events over distinct per-layer weights, and the CPU oracle timed
+on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # MI355X published HBM3E bandwidth, bytes/s
+
+
+def qweight_bytes(K, N):
+    sh = (K + 127) // 128
+    return N * (((K + 31) // 32) * 16 + ((sh + 7) // 8) * 4 + sh * 2)
+
+
+def weight_bytes_per_token(cfg):
+    dim, hid, L, V = cfg["dim"], cfg["hidden_dim"], cfg["n_layers"], cfg["vocab_size"]
+    kv_dim = dim * cfg["n_kv_heads"] // cfg["n_heads"]
+    layer = 2 * qweight_bytes(dim, dim) + 2 * qweight_bytes(dim, kv_dim) + 2 * qweight_bytes(dim, hid) + qweight_bytes(hid, dim) + 4 * dim
+    return L * layer + 2 * V * dim + 2 * dim + 2 * dim  # + classifier + final norm + one embedding row
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--config", default="7b", choices=["7b", "13b", "33b"])
+    ap.add_argument("--start-pos", type=int, default=0, help="pre-fill the KV cache with N(0,1) up to this position first")
+    ap.add_argument("--schedule", default="fused", choices=["fused", "reference"])
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--cpu-tokens", type=int, default=12, help="tokens of the same model timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the whole model on ONE GPU (no collectives); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+
+    import llama_cu_awq_amd as A
+    from llama_cu_awq_amd import synth
+
+    cfg = {"7b": synth.CONFIG_7B, "13b": synth.CONFIG_13B, "33b": synth.CONFIG_33B}[args.config]
+    n_prompt = max(1, args.warmup)
+    total = n_prompt + args.steps
+    assert args.start_pos + total <= cfg["seq_len"], "warmup + steps exceeds seq_len"
+    mode = A.SCHEDULE_FUSED if args.schedule == "fused" else A.SCHEDULE_REFERENCE
+    use_graph = not args.no_graph
+
+    t0 = time.time()
+    image = synth.make_model_image(cfg, seed=args.seed, threads=min(16, os.cpu_count() or 8))
+    print(f"[bench] model image {image.nbytes / 1e9:.2f} GB generated in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+    ctx = A.Context(0)
+    t0 = time.time()
+    model = A.Transformer(ctx, image=image)
+    print(f"[bench] uploaded in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+
+    vocab = cfg["vocab_size"]
+    kv_dim = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"]
+    prompt = synth.prompt_tokens(args.seed, n_prompt, vocab)
+    model.reset(prompt)
+    if args.start_pos:
+        # KV cache pre-filled with N(0,1) below start_pos (long-context configuration)
+        for name in ("key_cache", "value_cache"):
+            buf = model.buffer(name, cfg["n_layers"] * cfg["seq_len"] * kv_dim * 2)
+            for l in range(cfg["n_layers"]):
+                vals = synth.normal_f16(synth.stream_key(args.seed, name, l), args.start_pos * kv_dim)
+                buf.write(vals, offset_bytes=l * cfg["seq_len"] * kv_dim * 2)
+        model.set_pos(args.start_pos, prompt[0])
+        tok = (np.ctypeslib.as_array(model._tokens))
+        tok[args.start_pos : args.start_pos + n_prompt] = prompt
+
+    def step(i):
+        ctx.sync()  # the reference loop waits for the previous token before launching the next (llama2_q4.cu:713)
+        model.forward(gen_token=(i >= n_prompt - 1), use_graph=use_graph, mode=mode)
+
+    for i in range(n_prompt):  # warm-up: the prompt
+        step(i)
+    ctx.sync()
+    ev0, ev1 = ctx.event(), ctx.event()
+    ctx.record(ev0)
+    w0 = time.perf_counter()
+    for i in range(n_prompt, total):
+        step(i)
+    ctx.record(ev1)
+    ctx.sync()
+    wall = time.perf_counter() - w0
+    gpu_ms = ctx.elapsed_ms(ev0, ev1)
+    tok_s = args.steps / wall
+    first = args.start_pos + n_prompt
+    gen = [model.token(first + i) for i in range(min(8, args.steps))]
+
+    wbytes = weight_bytes_per_token(cfg)
+    avg_kv = 2 * cfg["n_layers"] * kv_dim * 2 * (args.start_pos + n_prompt + (args.steps + 1) / 2.0)
+    decode_gbps = (wbytes + avg_kv) * tok_s / 1e9
+
+    # ---- dominant kernel: fused gate/up int4 matvec + SiLU*mul, one launch per layer over that layer's own weights
+    dim, hid = cfg["dim"], cfg["hidden_dim"]
+    layers = [model.layer(l) for l in range(cfg["n_layers"])]
+    xb = model.buffer("xb", dim * 2)
+    hb = model.buffer("hb", hid * 2)
+    reps = 8
+
+    def ffn_pass():
+        for L in layers:
+            A.ffn_matvec_silu(ctx, hb, xb, L["wq_gate"], L["wq_up"], dim, hid)
+
+    ffn_pass()
+    ctx.sync()
+    ctx.record(ev0)
+    for _ in range(reps):
+        ffn_pass()
+    ctx.record(ev1)
+    ctx.sync()
+    ffn_us = ctx.elapsed_ms(ev0, ev1) * 1e3 / (reps * len(layers))
+    ffn_bytes = 2 * qweight_bytes(dim, hid) + dim * 2 + hid * 2
+    ffn_gbps = ffn_bytes / ffn_us / 1e3
+
+    # ---- the single 4096x4096-class GEMV (q/k/v/o shapes), rotating over every layer's four matrices
+    resid = model.buffer("x", dim * 2)
+
+    def gemv_pass():
+        for L in layers:
+            for n in ("wq_q", "wq_k", "wq_v", "wq_o"):
+                A.matmul_q(ctx, resid, xb, L[n], dim, dim)
+
+    gemv_pass()
+    ctx.sync()
+    ctx.record(ev0)
+    for _ in range(reps):
+        gemv_pass()
+    ctx.record(ev1)
+    ctx.sync()
+    gemv_us = ctx.elapsed_ms(ev0, ev1) * 1e3 / (reps * len(layers) * 4)
+    gemv_bytes = qweight_bytes(dim, dim) + 4 * dim
+    gemv_gbps = gemv_bytes / gemv_us / 1e3
+
+    # ---- CPU baseline: the oracle on the same model, a bounded number of tokens
+    cpu = None
+    if args.cpu_tokens > 0:
+        from oracle import oracle
+
+        o = oracle.Model(image)
+        o.reset(prompt)
+        o.forward(False)  # touch the weights once
+        c0 = time.perf_counter()
+        for _ in range(args.cpu_tokens):
+            o.forward(False)
+        cpu_s = time.perf_counter() - c0
+        cpu = {
+            "value": round(args.cpu_tokens / cpu_s, 4),
+            "unit": "tok/s",
+            "cores": oracle.num_threads(),
+            "kind": "port",
+            "sample": f"{args.cpu_tokens} tokens of the same {args.config} model (positions 1..{args.cpu_tokens}) through the scalar C++/OpenMP oracle, after 1 untimed token",
+        }
+        o.close()
+
+    out = {
+        "metric": "decode tok/s bs=1 @7B shape; int4 GEMV HBM GB/s vs ~8 TB/s peak",
+        "value": round(tok_s, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3 / args.steps, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int4 weights x fp16 activations, fp32 accumulate",
+        "data": "synthetic (random int4-g128 weights, fp16 scales, random prompt ids; seed %d)" % args.seed,
+        "config": {
+            "workload": f"llama-2-{args.config}-shape bs=1 greedy decode: {n_prompt}-token prompt then {args.steps} decode steps from position {args.start_pos}",
+            "schedule": args.schedule,
+            "graph": use_graph,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gemv_int4_kernel<2, FFN> (fused gate/up + SiLU*mul), K=%d N=%d" % (dim, hid),
+            "achieved": round(ffn_gbps, 1),
+            "peak": HBM_PEAK / 1e9,
+            "unit": "GB/s",
+            "frac": round(ffn_gbps * 1e9 / HBM_PEAK, 4),
+            "traffic": None,
+            "bytes_per_launch": ffn_bytes,
+            "us_per_launch": round(ffn_us, 3),
+        },
+        "cpu_baseline": cpu,
+        "decode": {
+            "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
+            "weight_bytes_per_token": wbytes,
+            "avg_kv_bytes_per_token": int(avg_kv),
+            "hbm_gbps": round(decode_gbps, 1),
+            "frac_of_weight_roofline": round(tok_s / (HBM_PEAK / wbytes), 4),
+            "first_tokens": gen,
+        },
+        "gemv_int4_%dx%d" % (dim, dim): {"us_per_launch": round(gemv_us, 3), "bytes": gemv_bytes, "gbps": round(gemv_gbps, 1), "frac": round(gemv_gbps * 1e9 / HBM_PEAK, 4)},
+    }
+    print(json.dumps(out), flush=True)
+    model.close()
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

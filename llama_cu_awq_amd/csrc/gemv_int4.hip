@@ -11,11 +11,12 @@
 // 32 consecutive K elements (one 16-byte load of packed weights, the same lane
 // ownership as the reference's uint4 load) meet their activations as packed
 // fp16 pairs.  Each wave owns R consecutive rows and walks the row in passes
-// of 64 x 16 bytes, with the next pass's loads issued before the current pass
-// is consumed; a lane keeps its activations in registers across the R rows.
-// Nibbles become fp16 integers with the 0x6400 mantissa trick, the zero point
-// is subtracted exactly in fp16, products are accumulated in fp32 by
-// v_dot2_f32_f16, and the group scale is applied once per 32 elements in fp32.
+// of 64 x 16 bytes; two passes of loads are kept in flight, the first two
+// requested before staging starts; a lane reads its activations from LDS once
+// per pass and reuses them for the R rows.  Nibbles become fp16 numbers by
+// OR-ing them into the mantissa of 1024.0, products are accumulated in fp32 by
+// v_dot2_f32_f16 with the 1024 offset and the zero point cancelled through
+// per-chunk constants, and the group scale is applied once per 32 elements.
 #include "common.hpp"
 
 namespace {
@@ -43,28 +44,28 @@ struct GemvParams {
 
 enum { KIND_SINGLE = 0, KIND_QKV = 1, KIND_FFN = 2 };
 
-// Sum over 32 consecutive K elements of (q - z) * x, exact products, fp32 sum.
-// w: 4 dwords of 8 nibbles; xq[qi]: the 8 activations of dword qi as pairs
-// (0,4) (1,5) (2,6) (3,7).
-__device__ __forceinline__ float chunk_dot(const u32x4 w, const uint32_t z, const u32x4 (&xq)[4]) {
-    // fp16 constants: -(1024 + z) and -(64 + z), both exactly representable
-    const h16x2 zlo = as_h2(0xE400E400u | (z * 0x00010001u));
-    const h16x2 zhi = as_h2(0xD400D400u | (z * 0x00100010u));
-    const h16x2 sixteenth = {(h16_t)0.0625f, (h16_t)0.0625f};
-    float acc = 0.0f;
+// sum over the 32 consecutive K elements of one chunk of (q - z) * x.
+//
+// w: 4 dwords of 8 nibbles.  xq[qi]: the 8 activations of dword qi as fp16 pairs
+// (x0,x4) (x1/16,x5/16) (x2,x6) (x3/16,x7/16).  OR-ing a nibble into the
+// mantissa of fp16 1024.0 gives 1024+q (nibble at bits 0-3) or 1024+16q (bits
+// 4-7) exactly, so
+//   sum_k (1024 + [16] q_k) * X_k  =  1024 * sum_k X_k  +  sum_k q_k x_k
+// and the chunk's constants A = sum x and B = 1024 * sum X (computed once when
+// x is staged) turn that into sum (q - z) x = dot - B - z*A.  The accumulator
+// starts at -B - z*A so that the large common term cancels first.  Products are
+// exact in fp32 (11-bit x 11-bit significands); only the fp32 additions round.
+__device__ __forceinline__ float chunk_dot(const u32x4 w, const float zf, const u32x4 (&xq)[4], const float A, const float B,
+                                           const uint32_t magic) {
+    float acc = fmaf(-zf, A, -B);
 #pragma unroll
     for (int qi = 0; qi < 4; qi++) {
         const uint32_t d = w[qi];
         const uint32_t d8 = d >> 8;
-        // 0x6400 | n  == 1024 + n ;  0x6400 | (n << 4) == 1024 + 16 n   (fp16, exact)
-        h16x2 t0 = as_h2((d & 0x000F000Fu) | 0x64006400u) + zlo;                                     // q0-z, q4-z
-        h16x2 t1 = __builtin_elementwise_fma(as_h2((d & 0x00F000F0u) | 0x64006400u), sixteenth, zhi);   // q1-z, q5-z
-        h16x2 t2 = as_h2((d8 & 0x000F000Fu) | 0x64006400u) + zlo;                                    // q2-z, q6-z
-        h16x2 t3 = __builtin_elementwise_fma(as_h2((d8 & 0x00F000F0u) | 0x64006400u), sixteenth, zhi);  // q3-z, q7-z
-        acc = __builtin_amdgcn_fdot2(t0, as_h2(xq[qi][0]), acc, false);
-        acc = __builtin_amdgcn_fdot2(t1, as_h2(xq[qi][1]), acc, false);
-        acc = __builtin_amdgcn_fdot2(t2, as_h2(xq[qi][2]), acc, false);
-        acc = __builtin_amdgcn_fdot2(t3, as_h2(xq[qi][3]), acc, false);
+        acc = dot2((d & 0x000F000Fu) | magic, xq[qi][0], acc);
+        acc = dot2((d & 0x00F000F0u) | magic, xq[qi][1], acc);
+        acc = dot2((d8 & 0x000F000Fu) | magic, xq[qi][2], acc);
+        acc = dot2((d8 & 0x00F000F0u) | magic, xq[qi][3], acc);
     }
     return acc;
 }
@@ -91,28 +92,31 @@ __device__ __forceinline__ void load_stage(Stage<NS>& st, const uint32_t* const 
 }
 
 template <int NS>
-__device__ __forceinline__ void consume_stage(const Stage<NS>& st, const u32x4* xs, int c, int C, float (&sum)[NS]) {
+__device__ __forceinline__ void consume_stage(const Stage<NS>& st, const u32x4* xs, const float2* ab, int c, int C,
+                                              float (&sum)[NS], const uint32_t magic) {
     if (c < C) {
         u32x4 xq[4];
 #pragma unroll
         for (int qi = 0; qi < 4; qi++) xq[qi] = xs[qi * C + c];
+        const float2 cab = ab[c];
         const int zshift = ((c >> 2) & 7) * 4;
 #pragma unroll
         for (int i = 0; i < NS; i++) {
-            const uint32_t z = (st.zw[i] >> zshift) & 0xFu;
-            const float acc = chunk_dot(st.w[i], z, xq);
+            const float zf = (float)((st.zw[i] >> zshift) & 0xFu);
+            const float acc = chunk_dot(st.w[i], zf, xq, cab.x, cab.y, magic);
             sum[i] = fmaf(half_bits_to_float(st.s[i]), acc, sum[i]);
         }
     }
 }
 
-// Stage x (K halves) into LDS as u32x4 words laid out [qi][chunk], each holding
-// the 8 activations of dword qi of that chunk as pairs (0,4)(1,5)(2,6)(3,7);
-// elements in [K, 32*C) are zero.  With NORM the vector is RMS-normalised on
-// the way in with the reference's arithmetic (gpu_kernels.h:72-105):
+// Stage x (K halves) into LDS: xs[qi*C + c] holds the 8 activations of dword qi
+// of chunk c as pairs (x0,x4)(x1/16,x5/16)(x2,x6)(x3/16,x7/16), and ab[c] =
+// {A, B} the chunk constants described at chunk_dot.  Elements in [K, 32*C)
+// are zero.  With NORM the vector is RMS-normalised on the way in with the
+// reference's arithmetic (gpu_kernels.h:72-105):
 // o = half(x * (rsqrt(mean(x^2) + 1e-5) * w)).
 template <bool NORM>
-__device__ __forceinline__ void stage_x(u32x4* xs, const GemvParams& p, float* red) {
+__device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const GemvParams& p, float* red) {
     const int tid = threadIdx.x;
     const int n8 = p.K >> 3;  // 8-half pieces of real data
     const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
@@ -140,7 +144,9 @@ __device__ __forceinline__ void stage_x(u32x4* xs, const GemvParams& p, float* r
     const u32x4* wg = reinterpret_cast<const u32x4*>(p.norm_w);
     u32x4* og = reinterpret_cast<u32x4*>(p.norm_out);
     const bool store_norm = NORM && og != nullptr && blockIdx.x == 0 && blockIdx.y == 0;
-    for (int e = tid; e < p.C * 4; e += 256) {
+    const h16x2 sixteenth = {(h16_t)0.0625f, (h16_t)0.0625f};
+    for (int e0 = 0; e0 < p.C * 4; e0 += 256) {  // uniform trip count: the quad reduction below needs all lanes
+        const int e = e0 + tid;
         u32x4 v = {0u, 0u, 0u, 0u};
         if (e < n8) {
             v = xg[e];
@@ -159,12 +165,24 @@ __device__ __forceinline__ void stage_x(u32x4* xs, const GemvParams& p, float* r
             }
         }
         // v holds halves h0..h7 as (h0,h1)(h2,h3)(h4,h5)(h6,h7) -> (h0,h4)(h1,h5)(h2,h6)(h3,h7)
-        u32x4 o;
-        o[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
-        o[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
-        o[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
-        o[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
-        xs[(e & 3) * p.C + (e >> 2)] = o;
+        const h16x2 p0 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x05040100u));
+        const h16x2 p1 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x07060302u)) * sixteenth;
+        const h16x2 p2 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x05040100u));
+        const h16x2 p3 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x07060302u)) * sixteenth;
+        const float even = ((float)p0[0] + (float)p0[1]) + ((float)p2[0] + (float)p2[1]);
+        const float odd = ((float)p1[0] + (float)p1[1]) + ((float)p3[0] + (float)p3[1]);
+        float a = fmaf(16.0f, odd, even);  // sum of the activations as the dot product sees them
+        float b = even + odd;              // sum of the stored fp16 values
+        // the 4 dword pieces of a chunk sit in 4 adjacent lanes
+        a += dpp_mov<0xB1>(a);
+        a += dpp_mov<0x4E>(a);
+        b += dpp_mov<0xB1>(b);
+        b += dpp_mov<0x4E>(b);
+        if (e < p.C * 4) {
+            u32x4 o = {as_u32(p0), as_u32(p1), as_u32(p2), as_u32(p3)};
+            xs[(e & 3) * p.C + (e >> 2)] = o;
+            if ((e & 3) == 0) ab[e >> 2] = make_float2(a, 1024.0f * b);
+        }
     }
     __syncthreads();
 }
@@ -173,15 +191,15 @@ template <int R, int KIND, bool NORM>
 __global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
     extern __shared__ u32x4 xs[];
     __shared__ float red[4];
-    stage_x<NORM>(xs, p, red);
-
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int C = p.C;
     const int pwh = C * 4;
+    float2* ab = reinterpret_cast<float2*>(xs + 4 * C);
     const int which = (KIND == KIND_QKV) ? blockIdx.y : 0;
-    const int row0 = (blockIdx.x * 4 + wave) * R;
-    if (row0 >= p.N) return;
+    const int row0 = min((blockIdx.x * 4 + wave) * R, p.N - 1);  // a wave past N recomputes the last row, stores nothing
+    uint32_t magic = 0x64006400u;  // fp16 pair (1024.0, 1024.0), kept in a VGPR
+    asm("" : "+v"(magic));
 
     constexpr int NS = (KIND == KIND_FFN) ? 2 * R : R;
     const uint32_t* wrow[NS];
@@ -209,20 +227,24 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
 #pragma unroll
     for (int i = 0; i < NS; i++) sum[i] = 0.0f;
 
+    // The first two passes of packed weights are requested before x is staged, so
+    // that their HBM latency overlaps the staging (and the RMSNorm reduction).
     Stage<NS> a, b;
     load_stage<NS>(a, wrow, zrow, srow, lane, C);
+    load_stage<NS>(b, wrow, zrow, srow, lane + 64, C);
+    stage_x<NORM>(xs, ab, p, red);
     for (int c = lane; c < C + lane; c += 128) {  // wave-uniform trip count
         const int c1 = c + 64;
-        load_stage<NS>(b, wrow, zrow, srow, c1, C);
-        consume_stage<NS>(a, xs, c, C, sum);
+        consume_stage<NS>(a, xs, ab, c, C, sum, magic);
         load_stage<NS>(a, wrow, zrow, srow, c1 + 64, C);
-        consume_stage<NS>(b, xs, c1, C, sum);
+        consume_stage<NS>(b, xs, ab, c1, C, sum, magic);
+        load_stage<NS>(b, wrow, zrow, srow, c1 + 128, C);
     }
 
 #pragma unroll
     for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]);
 
-    if (lane == 0) {
+    if (lane == 0 && (blockIdx.x * 4 + wave) * R < p.N) {
         uint16_t* out = (KIND == KIND_QKV) ? (which == 0 ? p.out[0] : (which == 1 ? p.out[1] : p.out[2])) : p.out[0];
         const int loff = (KIND == KIND_QKV) ? (which == 0 ? p.loff[0] : (which == 1 ? p.loff[1] : p.loff[2])) : p.loff[0];
         if (loff != -1) out += (size_t)loff + (size_t)(*p.pos) * p.N;
@@ -303,7 +325,7 @@ bool qw_ok(const awq_qweight* w) { return w && w->weight && w->zeros && w->scale
 template <int R, int KIND>
 int launch(awq_ctx* ctx, const GemvParams& p, int grid_y, const char* what) {
     const dim3 grid(div_up(p.N, 4 * R), grid_y);
-    const size_t lds = (size_t)p.C * 64;
+    const size_t lds = (size_t)p.C * 72;  // activations + per-chunk constants
     if (p.norm_w)
         hipLaunchKernelGGL((gemv_int4_kernel<R, KIND, true>), grid, dim3(256), lds, ctx->stream, p);
     else
