@@ -41,7 +41,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--config", default="7b", choices=["7b", "13b", "33b"])
     ap.add_argument("--start-pos", type=int, default=0, help="pre-fill the KV cache with N(0,1) up to this position first")
-    ap.add_argument("--schedule", default="fused", choices=["fused", "reference"])
+    ap.add_argument("--schedule", default="fused", choices=["persistent", "fused", "reference"])
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=12, help="tokens of the same model timed on the CPU oracle (0 = skip)")
     ap.add_argument("--seed", type=int, default=0)
@@ -59,7 +59,7 @@ def main():
     n_prompt = max(1, args.warmup)
     total = n_prompt + args.steps
     assert args.start_pos + total <= cfg["seq_len"], "warmup + steps exceeds seq_len"
-    mode = A.SCHEDULE_FUSED if args.schedule == "fused" else A.SCHEDULE_REFERENCE
+    mode = {"persistent": A.SCHEDULE_PERSISTENT, "fused": A.SCHEDULE_FUSED, "reference": A.SCHEDULE_REFERENCE}[args.schedule]
     use_graph = not args.no_graph
 
     t0 = time.time()

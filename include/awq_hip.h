@@ -181,10 +181,20 @@ int awq_transformer_set_pos(awq_transformer* t, int pos, int token);
  * use_graph != 0 replays a recorded launch sequence keyed by sequence-length bin (the USE_CUDA_GRAPHS path,
  * llama2_q4.cu:553-575); 0 launches eagerly.  mode selects the schedule: AWQ_SCHEDULE_REFERENCE issues the
  * reference's op sequence one launcher at a time; AWQ_SCHEDULE_FUSED merges RMSNorm into the consuming
- * matrix-vector kernels and RoPE into the QKV kernel (same rounding points). */
+ * matrix-vector kernels (same rounding points); AWQ_SCHEDULE_PERSISTENT runs the whole token, sampler included,
+ * as ONE launch of a persistent kernel (one workgroup per CU, grid barriers between the steps, weights prefetched
+ * across steps); it ignores use_graph and returns AWQ_ERR_SHAPE for models whose shape its work split cannot take
+ * (the other two schedules run every model). */
 #define AWQ_SCHEDULE_REFERENCE 0
 #define AWQ_SCHEDULE_FUSED 1
+#define AWQ_SCHEDULE_PERSISTENT 2
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode);
+
+/* Diagnostics of the persistent schedule (no counterpart in the reference; its DUMP_PER_TOKEN_TIMINGS switch,
+ * llama2_q4.cu:32, 545-600, times whole tokens only).  enable != 0 makes later persistent launches record, for
+ * workgroup 0, five 100-MHz wall-clock stamps per step (start, input staged, products done, results published,
+ * grid barrier passed); host_out (may be NULL) receives the stamps of the most recent launch first. */
+int awq_transformer_trace(awq_transformer* t, int enable, long long* host_out, int max_entries, int* nphases);
 
 #ifdef __cplusplus
 }

@@ -15,4 +15,4 @@ from .ops import (  # noqa: F401
     qkv_matvec,
     rmsnorm,
 )
-from .model import Transformer, SCHEDULE_FUSED, SCHEDULE_REFERENCE  # noqa: F401
+from .model import Transformer, SCHEDULE_FUSED, SCHEDULE_PERSISTENT, SCHEDULE_REFERENCE  # noqa: F401

@@ -76,6 +76,7 @@ PROTOTYPES = {
     "awq_transformer_reset": [_vp, C.POINTER(C.c_int), _i],
     "awq_transformer_set_pos": [_vp, _i, _i],
     "awq_transformer_forward": [_vp, _i, _i, _i],
+    "awq_transformer_trace": [_vp, _i, C.POINTER(C.c_longlong), _i, C.POINTER(C.c_int)],
 }
 NON_STATUS = {"awq_last_error": ([], C.c_char_p), "awq_ctx_stream": ([_vp], _vp)}
 

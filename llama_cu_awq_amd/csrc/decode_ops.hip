@@ -316,7 +316,7 @@ __global__ __launch_bounds__(256) void gemv_f16_kernel(uint16_t* out, const uint
 // One workgroup of 1024: per-thread strided scan keeping the first maximum,
 // then (value, index) reductions that prefer the lower index on equal values.
 __global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* x, int size, int* result, volatile int* pPos,
-                                                      int* pPosGpu, int write_token) {
+                                                      int* pPosGpu, int write_token, int* mirror) {
     __shared__ float red_v[16];
     __shared__ int red_i[16];
     const int tid = threadIdx.x;
@@ -352,7 +352,10 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* x, int siz
         if (best_i == 0x7FFFFFFF) best_i = 0;  // nothing compared greater than -inf (all NaN / -inf)
         int token_pos = *pPosGpu;
         token_pos++;
-        if (write_token) result[token_pos] = best_i;
+        if (write_token) {
+            result[token_pos] = best_i;
+            if (mirror) mirror[token_pos] = best_i;
+        }
         *pPos = token_pos;
         *pPosGpu = token_pos;
     }
@@ -376,6 +379,14 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
 }
 
 }  // namespace
+
+// Internal: greedy sampler that also records the token in a device-side mirror of the token list.
+int awq_launch_argmax(awq_ctx* ctx, const uint16_t* logits, int size, int* tokens, volatile int* pos_host, int* pos_dev,
+                      int write_token, int* tokens_mirror) {
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, ctx->stream, logits, size, tokens, pos_host, pos_dev, write_token,
+                       tokens_mirror);
+    return awq_check_launch("argmax");
+}
 
 // Internal: fp16 matvec with optional fused RMSNorm of x (norm_out must not alias x).
 int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
@@ -456,8 +467,7 @@ int awq_argmax_advance(awq_ctx* ctx, const uint16_t* logits, int size, int* toke
     if (int r = awq_bind(ctx)) return r;
     AWQ_REQUIRE(logits && tokens && pos_host && pos_dev, AWQ_ERR_ARG, "null pointer");
     AWQ_REQUIRE(size > 0, AWQ_ERR_SHAPE, "size must be positive");
-    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, ctx->stream, logits, size, tokens, pos_host, pos_dev, write_token);
-    return awq_check_launch("argmax");
+    return awq_launch_argmax(ctx, logits, size, tokens, pos_host, pos_dev, write_token, nullptr);
 }
 
 }  // extern "C"

@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include "token_kernel.hpp"
 
 int awq_launch_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* w, int K, int N, int accum,
                            int gpu_count, int loff, const int* pos, const uint16_t* norm_w, uint16_t* norm_out);
@@ -22,6 +23,8 @@ int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qwe
                    int N, const uint16_t* norm_w, uint16_t* norm_out);
 int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
                           const uint16_t* norm_w, uint16_t* norm_out);
+int awq_launch_argmax(awq_ctx* ctx, const uint16_t* logits, int size, int* tokens, volatile int* pos_host, int* pos_dev,
+                      int write_token, int* tokens_mirror);
 
 namespace {
 
@@ -48,6 +51,16 @@ struct awq_transformer {
     SharedData* shared;
     hipGraphExec_t graphs[2][kMaxGraphs];
     bool captured[2][kMaxGraphs];
+    int* tokens_dev;  // device mirror of SharedData.tokens (the persistent kernel reads its input token here)
+    // plan of the persistent per-token kernel
+    bool tk_ok;
+    char tk_why[160];  // why the persistent kernel cannot run this model, when !tk_ok
+    tk::Args tk_args;
+    size_t tk_lds_bytes;
+    tk::Phase* tk_phases;
+    tk::Sync* tk_sync;
+    int* tk_err_host;
+    long long* tk_trace;  // device buffer of per-phase time stamps when tracing is on, else null
 };
 
 namespace {
@@ -138,6 +151,8 @@ int alloc_state(awq_transformer* t) {
     AWQ_HIP_TRY(hipMemset(s.pos, 0, sizeof(int)));
     AWQ_HIP_TRY(hipHostMalloc((void**)&t->shared, sizeof(SharedData), hipHostMallocDefault));
     memset((void*)t->shared, 0, sizeof(SharedData));
+    AWQ_HIP_TRY(hipMalloc((void**)&t->tokens_dev, (size_t)(c.seq_len + 8) * sizeof(int)));
+    AWQ_HIP_TRY(hipMemset(t->tokens_dev, 0, (size_t)(c.seq_len + 8) * sizeof(int)));
     s.shared_pos = &t->shared->pos;
     s.shared_tokens = t->shared->tokens;
     return AWQ_OK;
@@ -159,6 +174,11 @@ void release(awq_transformer* t) {
     (void)hipFree(t->s.value_cache);
     (void)hipFree(t->s.pos);
     if (t->shared) (void)hipHostFree(t->shared);
+    (void)hipFree(t->tokens_dev);
+    (void)hipFree(t->tk_phases);
+    (void)hipFree(t->tk_sync);
+    (void)hipFree(t->tk_trace);
+    if (t->tk_err_host) (void)hipHostFree(t->tk_err_host);
     delete t;
 }
 
@@ -168,9 +188,184 @@ awq_transformer* new_transformer(awq_ctx* ctx) {
     t->blob = nullptr;
     t->blob_bytes = 0;
     t->shared = nullptr;
+    t->tokens_dev = nullptr;
+    t->tk_ok = false;
+    t->tk_why[0] = 0;
+    t->tk_phases = nullptr;
+    t->tk_sync = nullptr;
+    t->tk_err_host = nullptr;
+    t->tk_trace = nullptr;
     memset(&t->s, 0, sizeof(t->s));
     memset(t->captured, 0, sizeof(t->captured));
     return t;
+}
+
+
+// Plan the persistent per-token kernel for this model: choose the grid, lay out LDS, build the phase list.
+// Leaves t->tk_ok false (with the reason in t->tk_why) when the model's shape does not fit the kernel's
+// work split; the multi-kernel schedules still run such a model.
+#define TK_REQUIRE(cond, why)                                   \
+    do {                                                        \
+        if (!(cond)) {                                          \
+            snprintf(t->tk_why, sizeof(t->tk_why), "%s", why);  \
+            return AWQ_OK;                                      \
+        }                                                       \
+    } while (0)
+
+int plan_token_kernel(awq_transformer* t) {
+    const awq_config& c = t->cfg;
+    const int dim = c.dim, hidden = c.hidden_dim;
+    const int hs = dim / c.n_heads;
+    const int kv_dim = (dim * c.n_kv_heads) / c.n_heads;
+    hipDeviceProp_t prop;
+    AWQ_HIP_TRY(hipGetDeviceProperties(&prop, t->ctx->device));
+    int G = prop.multiProcessorCount < tk::kMaxWorkgroups ? prop.multiProcessorCount : tk::kMaxWorkgroups;
+    // every workgroup takes the same number of rows of every matrix
+    while (G >= 32 && !((dim / 2) % G == 0 && (kv_dim / 2) % G == 0 && hidden % G == 0)) G--;
+    TK_REQUIRE(G >= 32, "no grid size divides dim/2, kv_dim/2 and hidden_dim");
+    TK_REQUIRE(c.n_heads <= G, "more heads than workgroups");
+    TK_REQUIRE(hs == 64 || hs == 128 || hs == 256, "head size must be 64, 128 or 256");
+    TK_REQUIRE((scales_height(dim) & 1) == 0 && (scales_height(hidden) & 1) == 0, "odd number of groups per row");
+    TK_REQUIRE(dim <= 20480 && hidden <= 20480, "reduction length above 20480");
+    const int ppw = dim / 2 / G, kpw = kv_dim / 2 / G, vpw = kv_dim / G;
+    TK_REQUIRE(ppw + kpw + vpw <= 256 && 2 * hidden / G <= 512 && dim / G <= 256, "too many rows per workgroup");
+    const int cls_rows = div_up(c.vocab_size, G);
+    TK_REQUIRE(cls_rows <= 256, "too many classifier rows per workgroup");
+
+    auto passes = [](int K) { return div_up(div_up(K, 32), 64); };
+    const int cls_passes = div_up(dim / 8, 64);
+    int max_units = 1024;  // attention borrows 4 x 256 floats of this area
+    auto upd = [&](int v) { if (v > max_units) max_units = v; };
+    upd((2 * ppw + 2 * kpw + vpw) * passes(dim));
+    upd((dim / G) * passes(dim));
+    upd((2 * hidden / G) * passes(dim));
+    upd((dim / G) * passes(hidden));
+    upd(cls_rows * cls_passes);
+    const int cmax = div_up(dim > hidden ? dim : hidden, 32);
+    int xs_bytes = cmax * 64;
+    if (dim * 2 > xs_bytes) xs_bytes = dim * 2;
+    if (c.seq_len * 4 > xs_bytes) xs_bytes = c.seq_len * 4;
+    xs_bytes = (xs_bytes + 255) & ~255;
+    const int ab_bytes = (cmax * 8 + 255) & ~255;
+    const int part_bytes = (max_units * 4 + 255) & ~255;
+    const int misc_bytes = 1024;
+    const int lds_total = 160 * 1024;
+    const int fixed = xs_bytes + ab_bytes + part_bytes + misc_bytes;
+    int depth = (lds_total - fixed) / (tk::NSW * tk::UNIT_BYTES);
+    if (depth > 16) depth = 16;
+    TK_REQUIRE(depth >= 4, "not enough LDS left for the weight ring");
+
+    std::vector<tk::Phase> ph;
+    auto int4_phase = [&](int kind, int in_sel, int K, int N, int rows_per_wg, const uint16_t* norm_w, long long kvoff) {
+        tk::Phase p;
+        memset(&p, 0, sizeof(p));
+        p.kind = kind;
+        p.in_sel = in_sel;
+        p.K = K;
+        p.C = div_up(K, 32);
+        p.P = div_up(p.C, 64);
+        p.N = N;
+        p.rows_per_wg = rows_per_wg;
+        p.pzh = packed_zeros_height(K);
+        p.sh = scales_height(K);
+        p.kv_layer_off = kvoff;
+        p.norm_w = norm_w;
+        return p;
+    };
+    auto set_mat = [](tk::Phase& p, int i, const awq_qweight& w) {
+        p.w[i] = w.weight;
+        p.z[i] = w.zeros;
+        p.s[i] = w.scales;
+    };
+    for (int l = 0; l < c.n_layers; l++) {
+        const awq_layer_weights& L = t->layers[l];
+        const long long kvoff = (long long)l * c.seq_len * kv_dim;
+        tk::Phase q = int4_phase(tk::KIND_QKV, l == 0 ? tk::IN_EMBED : tk::IN_X, dim, dim, 2 * ppw + 2 * kpw + vpw, L.rms_att_weight, kvoff);
+        q.ppw = ppw;
+        q.kpw = kpw;
+        q.vpw = vpw;
+        set_mat(q, 0, L.wq_q);
+        set_mat(q, 1, L.wq_k);
+        set_mat(q, 2, L.wq_v);
+        ph.push_back(q);
+        tk::Phase at;
+        memset(&at, 0, sizeof(at));
+        at.kind = tk::KIND_ATTN;
+        at.kv_layer_off = kvoff;
+        ph.push_back(at);
+        tk::Phase o = int4_phase(tk::KIND_OPROJ, tk::IN_XB, dim, dim, dim / G, nullptr, kvoff);
+        set_mat(o, 0, L.wq_o);
+        ph.push_back(o);
+        tk::Phase f = int4_phase(tk::KIND_FFN, tk::IN_X, dim, hidden, 2 * hidden / G, L.rms_ffn_weight, kvoff);
+        set_mat(f, 0, L.wq_gate);
+        set_mat(f, 1, L.wq_up);
+        ph.push_back(f);
+        tk::Phase d = int4_phase(tk::KIND_DOWN, tk::IN_HB, hidden, dim, dim / G, nullptr, kvoff);
+        set_mat(d, 0, L.wq_down);
+        ph.push_back(d);
+    }
+    tk::Phase cl;
+    memset(&cl, 0, sizeof(cl));
+    cl.kind = tk::KIND_CLS;
+    cl.in_sel = tk::IN_X;
+    cl.K = dim;
+    cl.C = 0;
+    cl.P = cls_passes;
+    cl.N = c.vocab_size;
+    cl.rows_per_wg = cls_rows;
+    cl.w[0] = reinterpret_cast<const uint32_t*>(t->wcls);
+    cl.norm_w = t->rms_final;
+    ph.push_back(cl);
+    tk::Phase am;
+    memset(&am, 0, sizeof(am));
+    am.kind = tk::KIND_ARGMAX;
+    ph.push_back(am);
+
+    AWQ_HIP_TRY(hipMalloc((void**)&t->tk_phases, ph.size() * sizeof(tk::Phase)));
+    AWQ_HIP_TRY(hipMemcpy(t->tk_phases, ph.data(), ph.size() * sizeof(tk::Phase), hipMemcpyHostToDevice));
+    AWQ_HIP_TRY(hipMalloc((void**)&t->tk_sync, sizeof(tk::Sync)));
+    AWQ_HIP_TRY(hipMemset(t->tk_sync, 0, sizeof(tk::Sync)));
+    AWQ_HIP_TRY(hipHostMalloc((void**)&t->tk_err_host, sizeof(int), hipHostMallocDefault));
+    *t->tk_err_host = 0;
+
+    tk::Args& a = t->tk_args;
+    memset(&a, 0, sizeof(a));
+    a.phases = t->tk_phases;
+    a.nphases = (int)ph.size();
+    a.G = G;
+    a.depth = depth;
+    a.dim = dim;
+    a.hidden = hidden;
+    a.n_heads = c.n_heads;
+    a.n_kv_heads = c.n_kv_heads;
+    a.head_size = hs;
+    a.half_head_shift = hs == 64 ? 5 : (hs == 128 ? 6 : 7);
+    a.vocab = c.vocab_size;
+    a.rope_theta = c.rope_theta;
+    a.x = t->s.x;
+    a.xb = t->s.xb;
+    a.hb = t->s.hb;
+    a.q = t->s.q;
+    a.logits = t->s.logits;
+    a.key_cache = t->s.key_cache;
+    a.value_cache = t->s.value_cache;
+    a.embed = t->embed;
+    a.pos_dev = t->s.pos;
+    a.pos_host = t->s.shared_pos;
+    a.tokens_host = t->s.shared_tokens;
+    a.tokens_dev = t->tokens_dev;
+    a.sync = t->tk_sync;
+    a.err_host = t->tk_err_host;
+    a.spin_limit = 50000000LL;  // 0.5 s of the 100 MHz wall clock
+    if (const char* e = getenv("AWQ_TK_SPIN_LIMIT")) a.spin_limit = atoll(e);
+    a.lds_xs = 0;
+    a.lds_ab = xs_bytes;
+    a.lds_part = a.lds_ab + ab_bytes;
+    a.lds_misc = a.lds_part + part_bytes;
+    a.lds_ring = a.lds_misc + misc_bytes;
+    t->tk_lds_bytes = (size_t)a.lds_ring + (size_t)tk::NSW * depth * tk::UNIT_BYTES;
+    t->tk_ok = true;
+    return AWQ_OK;
 }
 
 // One token, the reference's launcher sequence with gpu_count = 1.
@@ -287,6 +482,7 @@ int awq_transformer_load_image(awq_ctx* ctx, const void* image, size_t bytes, aw
     }
     map_tensors(t);
     r = alloc_state(t);
+    if (r == AWQ_OK) r = plan_token_kernel(t);
     if (r) {
         release(t);
         return r;
@@ -369,6 +565,7 @@ int awq_transformer_load_file(awq_ctx* ctx, const char* checkpoint_path, awq_tra
     }
     map_tensors(t);
     r = alloc_state(t);
+    if (r == AWQ_OK) r = plan_token_kernel(t);
     if (r) {
         release(t);
         return r;
@@ -421,6 +618,9 @@ int awq_transformer_reset(awq_transformer* t, const int* prompt_tokens, int num_
     AWQ_HIP_TRY(hipMemset(t->s.pos, 0, sizeof(int)));
     t->shared->pos = 0;
     memcpy(t->shared->tokens, prompt_tokens, sizeof(int) * (size_t)num_prompt_tokens);
+    AWQ_HIP_TRY(hipMemcpy(t->tokens_dev, prompt_tokens, sizeof(int) * (size_t)num_prompt_tokens, hipMemcpyHostToDevice));
+    if (t->tk_err_host) *t->tk_err_host = 0;
+    if (t->tk_sync) AWQ_HIP_TRY(hipMemset(&t->tk_sync->error, 0, sizeof(int)));
     return AWQ_OK;
 }
 
@@ -432,14 +632,53 @@ int awq_transformer_set_pos(awq_transformer* t, int pos, int token) {
     AWQ_HIP_TRY(hipMemcpy(t->s.pos, &pos, sizeof(int), hipMemcpyHostToDevice));
     t->shared->pos = pos;
     t->shared->tokens[pos] = token;
+    AWQ_HIP_TRY(hipMemcpy(t->tokens_dev + pos, &token, sizeof(int), hipMemcpyHostToDevice));
+    return AWQ_OK;
+}
+
+int awq_transformer_trace(awq_transformer* t, int enable, long long* host_out, int max_entries, int* nphases) {
+    AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
+    if (int r = awq_bind(t->ctx)) return r;
+    AWQ_REQUIRE(t->tk_ok, AWQ_ERR_SHAPE, "persistent schedule unavailable for this model");
+    const size_t n = (size_t)t->tk_args.nphases * 5;
+    if (nphases) *nphases = t->tk_args.nphases;
+    if (host_out && t->tk_trace) {
+        AWQ_HIP_TRY(hipStreamSynchronize(t->ctx->stream));
+        const size_t m = n < (size_t)max_entries ? n : (size_t)max_entries;
+        AWQ_HIP_TRY(hipMemcpy(host_out, t->tk_trace, m * sizeof(long long), hipMemcpyDeviceToHost));
+    }
+    if (enable && !t->tk_trace) {
+        AWQ_HIP_TRY(hipMalloc((void**)&t->tk_trace, n * sizeof(long long)));
+        AWQ_HIP_TRY(hipMemset(t->tk_trace, 0, n * sizeof(long long)));
+    } else if (!enable && t->tk_trace) {
+        AWQ_HIP_TRY(hipStreamSynchronize(t->ctx->stream));
+        AWQ_HIP_TRY(hipFree(t->tk_trace));
+        t->tk_trace = nullptr;
+    }
     return AWQ_OK;
 }
 
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode) {
     AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
-    AWQ_REQUIRE(mode == AWQ_SCHEDULE_REFERENCE || mode == AWQ_SCHEDULE_FUSED, AWQ_ERR_ARG, "unknown schedule");
+    AWQ_REQUIRE(mode == AWQ_SCHEDULE_REFERENCE || mode == AWQ_SCHEDULE_FUSED || mode == AWQ_SCHEDULE_PERSISTENT, AWQ_ERR_ARG,
+                "unknown schedule");
     awq_ctx* ctx = t->ctx;
     if (int r = awq_bind(ctx)) return r;
+    if (mode == AWQ_SCHEDULE_PERSISTENT) {
+        if (!t->tk_ok) {
+            awq_set_error("persistent schedule unavailable for this model: %s", t->tk_why);
+            return AWQ_ERR_SHAPE;
+        }
+        if (*t->tk_err_host) {
+            awq_set_error("persistent kernel: a grid barrier timed out (workgroups not co-resident?)");
+            return AWQ_ERR_HIP;
+        }
+        AWQ_REQUIRE(t->shared->pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+        tk::Args a = t->tk_args;
+        a.write_token = gen_token;
+        a.trace = t->tk_trace;
+        return tk_launch(ctx->stream, a, t->tk_lds_bytes);
+    }
     // llama2_q4.cu:552: the host's view of the position sizes the attention launch
     const int seq_len = t->shared->pos + 1;
     AWQ_REQUIRE(seq_len <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
@@ -456,7 +695,7 @@ int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, in
             AWQ_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
             r = network(t, seq_len_bin, mode);
             if (r == AWQ_OK)
-                r = awq_argmax_advance(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, 1);
+                r = awq_launch_argmax(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, 1, t->tokens_dev);
             hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
             if (r) {
                 if (graph) (void)hipGraphDestroy(graph);
@@ -481,7 +720,7 @@ int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, in
         r = network(t, seq_len, mode);
     }
     if (r) return r;
-    return awq_argmax_advance(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token);
+    return awq_launch_argmax(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token, t->tokens_dev);
 }
 
 }  // extern "C"

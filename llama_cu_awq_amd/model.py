@@ -8,6 +8,7 @@ from .ops import DeviceBuffer, QWeight
 
 SCHEDULE_REFERENCE = 0
 SCHEDULE_FUSED = 1
+SCHEDULE_PERSISTENT = 2
 EOS_TOKEN = 2  # tokenizer.h:10
 
 

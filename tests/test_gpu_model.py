@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 TINY = dict(dim=256, hidden_dim=768, n_layers=2, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=64, rope_theta=10000.0)
 SMALL = dict(dim=1024, hidden_dim=2752, n_layers=4, n_heads=8, n_kv_heads=8, vocab_size=4096, seq_len=160, rope_theta=10000.0)
-GQA = dict(dim=512, hidden_dim=1376, n_layers=2, n_heads=8, n_kv_heads=2, vocab_size=1024, seq_len=64, rope_theta=10000.0)
+GQA = dict(dim=512, hidden_dim=1536, n_layers=2, n_heads=8, n_kv_heads=2, vocab_size=1024, seq_len=64, rope_theta=10000.0)
 
 
 @pytest.fixture(scope="module", params=["tiny", "small", "gqa"])
@@ -35,7 +35,7 @@ def test_header_round_trip(pair):
         assert t.config[k] == cfg[k] == o.config[k]
 
 
-@pytest.mark.parametrize("mode", [A.SCHEDULE_REFERENCE, A.SCHEDULE_FUSED])
+@pytest.mark.parametrize("mode", [A.SCHEDULE_REFERENCE, A.SCHEDULE_FUSED, A.SCHEDULE_PERSISTENT])
 def test_one_token_state(pair, mode):
     cfg, t, o = pair
     prompt = synth.prompt_tokens(1, 4, cfg["vocab_size"])
@@ -53,7 +53,7 @@ def test_one_token_state(pair, mode):
         assert rel_l2(got, want) <= 1e-2, name
 
 
-@pytest.mark.parametrize("mode,graph", [(A.SCHEDULE_REFERENCE, False), (A.SCHEDULE_FUSED, False), (A.SCHEDULE_FUSED, True), (A.SCHEDULE_REFERENCE, True)])
+@pytest.mark.parametrize("mode,graph", [(A.SCHEDULE_REFERENCE, False), (A.SCHEDULE_FUSED, False), (A.SCHEDULE_FUSED, True), (A.SCHEDULE_REFERENCE, True), (A.SCHEDULE_PERSISTENT, False)])
 def test_greedy_decode_matches_oracle(pair, mode, graph):
     cfg, t, o = pair
     n_prompt, steps = 8, min(48, cfg["seq_len"] - 1)
@@ -108,3 +108,32 @@ def test_load_file_equals_image(ctx, tmp_path):
     assert ta == tb
     a.close()
     b.close()
+
+
+def test_persistent_schedule_rejects_unsupported_shape(ctx):
+    """hidden_dim 1376 has an odd number of groups per row: the persistent kernel declines, the others run."""
+    cfg = dict(dim=512, hidden_dim=1376, n_layers=1, n_heads=4, n_kv_heads=4, vocab_size=512, seq_len=32, rope_theta=10000.0)
+    t = A.Transformer(ctx, image=synth.make_model_image(cfg, seed=5))
+    t.reset([5, 6])
+    with pytest.raises(A.AwqError) as e:
+        t.forward(False, False, A.SCHEDULE_PERSISTENT)
+    assert e.value.code == -2
+    t.forward(False, False, A.SCHEDULE_FUSED)
+    t.ctx.sync()
+    assert t.pos == 1
+    t.close()
+
+
+def test_schedules_can_be_mixed_within_a_sequence(pair):
+    """Tokens and positions stay consistent when consecutive tokens use different schedules."""
+    cfg, t, o = pair
+    prompt = synth.prompt_tokens(7, 4, cfg["vocab_size"])
+    want, _, _ = o.generate(prompt, 24, ignore_eos=True)
+    t.reset(prompt)
+    modes = [A.SCHEDULE_PERSISTENT, A.SCHEDULE_FUSED, A.SCHEDULE_REFERENCE]
+    for pos in range(24):
+        t.ctx.sync()
+        t.forward(pos >= len(prompt) - 1, False, modes[pos % 3])
+    t.ctx.sync()
+    got = [t.token(i) for i in range(25)]
+    assert got == want
