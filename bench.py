@@ -45,6 +45,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=12, help="tokens of the same model timed on the CPU oracle (0 = skip)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--only-kernels", action="store_true", help="skip the decode loop: run only the per-kernel loops and a 256 MiB device copy (for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the whole model on ONE GPU (no collectives); run with --gpus 1", file=sys.stderr)
@@ -89,10 +90,21 @@ def main():
         ctx.sync()  # the reference loop waits for the previous token before launching the next (llama2_q4.cu:713)
         model.forward(gen_token=(i >= n_prompt - 1), use_graph=use_graph, mode=mode)
 
+    ev0, ev1 = ctx.event(), ctx.event()
+    if args.only_kernels:
+        # calibration for HBM counters: a device-to-device copy of known size (reads 256 MiB, writes 256 MiB)
+        from llama_cu_awq_amd._lib import check, lib
+
+        nbytes = 256 << 20
+        src, dst = ctx.alloc(nbytes), ctx.alloc(nbytes)
+        check(lib.awq_memset_async(ctx.h, src.ptr, 1, nbytes))
+        for _ in range(4):
+            check(lib.awq_memcpy_d2d_async(ctx.h, dst.ptr, src.ptr, nbytes))
+        ctx.sync()
+        args.steps, n_prompt, total = 1, 1, 2
     for i in range(n_prompt):  # warm-up: the prompt
         step(i)
     ctx.sync()
-    ev0, ev1 = ctx.event(), ctx.event()
     ctx.record(ev0)
     w0 = time.perf_counter()
     for i in range(n_prompt, total):
@@ -196,7 +208,8 @@ def main():
             "peak": HBM_PEAK / 1e9,
             "unit": "GB/s",
             "frac": round(ffn_gbps * 1e9 / HBM_PEAK, 4),
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE (7B shape; profiles/gemv_int4_ffn_7b_pmc.md)
+            "traffic": 47048704 if (dim, hid) == (4096, 11008) else None,
             "bytes_per_launch": ffn_bytes,
             "us_per_launch": round(ffn_us, 3),
         },

@@ -70,6 +70,7 @@ int awq_free_host(awq_ctx* ctx, void* ptr);
 int awq_memcpy_h2d_async(awq_ctx* ctx, void* dst, const void* src, size_t bytes);
 int awq_memcpy_h2d(awq_ctx* ctx, void* dst, const void* src, size_t bytes); /* blocking */
 int awq_memcpy_d2h(awq_ctx* ctx, void* dst, const void* src, size_t bytes); /* blocking, ordered after the stream */
+int awq_memcpy_d2d_async(awq_ctx* ctx, void* dst, const void* src, size_t bytes);
 int awq_memset_async(awq_ctx* ctx, void* dst, int value, size_t bytes);
 
 /* ---- timing on the context's stream (cudaEvent pair, llama2_q4.cu:545-550, 592-600). */

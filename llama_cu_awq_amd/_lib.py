@@ -51,6 +51,7 @@ PROTOTYPES = {
     "awq_memcpy_h2d_async": [_vp, _vp, _vp, _sz],
     "awq_memcpy_h2d": [_vp, _vp, _vp, _sz],
     "awq_memcpy_d2h": [_vp, _vp, _vp, _sz],
+    "awq_memcpy_d2d_async": [_vp, _vp, _vp, _sz],
     "awq_memset_async": [_vp, _vp, _i, _sz],
     "awq_event_create": [_vp, _pvp],
     "awq_event_destroy": [_vp, _vp],

@@ -127,6 +127,12 @@ int awq_memcpy_d2h(awq_ctx* ctx, void* dst, const void* src, size_t bytes) {
     return AWQ_OK;
 }
 
+int awq_memcpy_d2d_async(awq_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return AWQ_OK;
+}
+
 int awq_memset_async(awq_ctx* ctx, void* dst, int value, size_t bytes) {
     if (int r = awq_bind(ctx)) return r;
     AWQ_HIP_TRY(hipMemsetAsync(dst, value, bytes, ctx->stream));

@@ -692,7 +692,7 @@ int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, in
         if (seq_len > seq_len_bin || graph_index == kMaxGraphs - 1 || seq_len_bin > t->cfg.seq_len) seq_len_bin = t->cfg.seq_len;
         if (!t->captured[mode][graph_index]) {
             hipGraph_t graph = nullptr;
-            AWQ_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+            AWQ_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
             r = network(t, seq_len_bin, mode);
             if (r == AWQ_OK)
                 r = awq_launch_argmax(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, 1, t->tokens_dev);
