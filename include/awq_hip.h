@@ -191,6 +191,21 @@ int awq_transformer_set_pos(awq_transformer* t, int pos, int token);
 #define AWQ_SCHEDULE_PERSISTENT 2
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode);
 
+/* ---- multi-token prefill.  No counterpart in the reference, which consumes the prompt one token per forward pass
+ * (llama2_q4.cu:716-735); the contract is the state that loop would leave. ---- */
+
+/* out[m*ldo + n] = half(sum_k a[m*lda + k] * W[n][k]) for M rows at once on the fp16 matrix cores, the weights
+ * dequantised to fp16 exactly as awq_dequant does; accum != 0 adds the previous contents of out (fused residual).
+ * K multiple of 32, N multiple of 128, lda multiple of 8. */
+int awq_gemm_int4(awq_ctx* ctx, uint16_t* out, int ldo, const uint16_t* a, int lda, int M, const awq_qweight* w, int K, int N,
+                  int accum);
+
+/* Consume the n_tokens tokens at positions pos .. pos+n_tokens-1 of the shared token list in one batched pass:
+ * afterwards the KV cache rows, the logits (of the last token), the token list and the position are those that
+ * n_tokens calls of awq_transformer_forward (gen_token false for all but the last, `gen_token` for the last) would
+ * leave.  Needs dim, kv_dim and hidden_dim to be multiples of 128.  Synchronises the stream on entry. */
+int awq_transformer_prefill(awq_transformer* t, int n_tokens, int gen_token);
+
 /* Diagnostics of the persistent schedule (no counterpart in the reference; its DUMP_PER_TOKEN_TIMINGS switch,
  * llama2_q4.cu:32, 545-600, times whole tokens only).  enable != 0 makes later persistent launches record, for
  * workgroup 0, five 100-MHz wall-clock stamps per step (start, input staged, products done, results published,

@@ -10,6 +10,7 @@ from .ops import (  # noqa: F401
     copy_embedding,
     dequant,
     ffn_matvec_silu,
+    gemm_q,
     matmul,
     matmul_q,
     qkv_matvec,

@@ -77,6 +77,8 @@ PROTOTYPES = {
     "awq_transformer_reset": [_vp, C.POINTER(C.c_int), _i],
     "awq_transformer_set_pos": [_vp, _i, _i],
     "awq_transformer_forward": [_vp, _i, _i, _i],
+    "awq_gemm_int4": [_vp, _vp, _i, _vp, _i, _i, _pq, _i, _i, _i],
+    "awq_transformer_prefill": [_vp, _i, _i],
     "awq_transformer_trace": [_vp, _i, C.POINTER(C.c_longlong), _i, C.POINTER(C.c_int)],
 }
 NON_STATUS = {"awq_last_error": ([], C.c_char_p), "awq_ctx_stream": ([_vp], _vp)}

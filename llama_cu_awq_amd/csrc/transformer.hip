@@ -25,6 +25,21 @@ int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const 
                           const uint16_t* norm_w, uint16_t* norm_out);
 int awq_launch_argmax(awq_ctx* ctx, const uint16_t* logits, int size, int* tokens, volatile int* pos_host, int* pos_dev,
                       int write_token, int* tokens_mirror);
+// prefill.hip
+int awq_launch_gemm_single(awq_ctx* ctx, uint16_t* out, long long ldo, const uint16_t* A, int lda, int M, const awq_qweight* w,
+                           int K, int N, int accum);
+int awq_launch_gemm_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, long long kv_row0_off,
+                        const uint16_t* A, int lda, int M, const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw,
+                        int K, int Nq, int Nkv);
+int awq_launch_gemm_ffn(awq_ctx* ctx, uint16_t* hb, const uint16_t* A, int lda, int M, const awq_qweight* gate_w,
+                        const awq_qweight* up_w, int K, int N);
+int awq_launch_embed_rows(awq_ctx* ctx, uint16_t* x, const uint16_t* table, int dim, const int* tokens, int pos0, int M);
+int awq_launch_rmsnorm_rows(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const uint16_t* w, int size, int M);
+int awq_launch_rope_rows(awq_ctx* ctx, uint16_t* q, uint16_t* kcache_layer, int nh, int nkv, int hs, int pos0, float theta, int M);
+int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, const uint16_t* kc, const uint16_t* vc, int nh, int hs,
+                            int kv_mul, int M, int pos0);
+int awq_launch_set_pos(awq_ctx* ctx, int* pos_dev, volatile int* pos_host, int value);
+int awq_launch_copy_row(awq_ctx* ctx, uint16_t* dst, const uint16_t* src, int n);
 
 namespace {
 
@@ -61,6 +76,9 @@ struct awq_transformer {
     tk::Sync* tk_sync;
     int* tk_err_host;
     long long* tk_trace;  // device buffer of per-phase time stamps when tracing is on, else null
+    // prefill workspace: activations of up to pf_rows tokens
+    int pf_rows;
+    uint16_t *pf_x, *pf_xb, *pf_q, *pf_att, *pf_hb;
 };
 
 namespace {
@@ -178,6 +196,11 @@ void release(awq_transformer* t) {
     (void)hipFree(t->tk_phases);
     (void)hipFree(t->tk_sync);
     (void)hipFree(t->tk_trace);
+    (void)hipFree(t->pf_x);
+    (void)hipFree(t->pf_xb);
+    (void)hipFree(t->pf_q);
+    (void)hipFree(t->pf_att);
+    (void)hipFree(t->pf_hb);
     if (t->tk_err_host) (void)hipHostFree(t->tk_err_host);
     delete t;
 }
@@ -195,6 +218,8 @@ awq_transformer* new_transformer(awq_ctx* ctx) {
     t->tk_sync = nullptr;
     t->tk_err_host = nullptr;
     t->tk_trace = nullptr;
+    t->pf_rows = 0;
+    t->pf_x = t->pf_xb = t->pf_q = t->pf_att = t->pf_hb = nullptr;
     memset(&t->s, 0, sizeof(t->s));
     memset(t->captured, 0, sizeof(t->captured));
     return t;
@@ -636,6 +661,69 @@ int awq_transformer_set_pos(awq_transformer* t, int pos, int token) {
     return AWQ_OK;
 }
 
+
+int awq_transformer_prefill(awq_transformer* t, int n_tokens, int gen_token) {
+    AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
+    awq_ctx* ctx = t->ctx;
+    if (int r = awq_bind(ctx)) return r;
+    const awq_config& p = t->cfg;
+    const int dim = p.dim, hidden = p.hidden_dim;
+    const int hs = dim / p.n_heads;
+    const int kv_dim = (dim * p.n_kv_heads) / p.n_heads;
+    const int kv_mul = p.n_heads / p.n_kv_heads;
+    AWQ_REQUIRE(n_tokens >= 1, AWQ_ERR_ARG, "n_tokens must be >= 1");
+    if ((dim & 127) || (kv_dim & 127) || (hidden & 127)) {
+        awq_set_error("prefill needs dim, kv_dim and hidden_dim to be multiples of 128 (got %d, %d, %d)", dim, kv_dim, hidden);
+        return AWQ_ERR_SHAPE;
+    }
+    AWQ_HIP_TRY(hipStreamSynchronize(ctx->stream));  // the host's view of the position must be current
+    const int pos_start = t->shared->pos;
+    AWQ_REQUIRE(pos_start + n_tokens <= p.seq_len, AWQ_ERR_ARG, "prompt runs past seq_len");
+    const int chunk = 512;
+    if (t->pf_rows == 0) {
+        const int rows = p.seq_len < chunk ? p.seq_len : chunk;
+        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_x, (size_t)rows * dim * 2));
+        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_xb, (size_t)rows * dim * 2));
+        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_q, (size_t)rows * dim * 2));
+        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_att, (size_t)rows * dim * 2));
+        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_hb, (size_t)rows * hidden * 2));
+        t->pf_rows = rows;
+    }
+    int r;
+    for (int done = 0; done < n_tokens; done += t->pf_rows) {
+        const int M = (n_tokens - done < t->pf_rows) ? n_tokens - done : t->pf_rows;
+        const int pos0 = pos_start + done;
+        if ((r = awq_launch_embed_rows(ctx, t->pf_x, t->embed, dim, t->tokens_dev, pos0, M))) return r;
+        for (int l = 0; l < p.n_layers; l++) {
+            const awq_layer_weights& L = t->layers[l];
+            const long long loff = (long long)l * p.seq_len * kv_dim;
+            if ((r = awq_launch_rmsnorm_rows(ctx, t->pf_xb, t->pf_x, L.rms_att_weight, dim, M))) return r;
+            if ((r = awq_launch_gemm_qkv(ctx, t->pf_q, t->s.key_cache, t->s.value_cache, loff + (long long)pos0 * kv_dim, t->pf_xb,
+                                         dim, M, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, kv_dim)))
+                return r;
+            if ((r = awq_launch_rope_rows(ctx, t->pf_q, t->s.key_cache + loff, p.n_heads, p.n_kv_heads, hs, pos0, p.rope_theta, M)))
+                return r;
+            if ((r = awq_launch_attn_prefill(ctx, t->pf_att, t->pf_q, t->s.key_cache + loff, t->s.value_cache + loff, p.n_heads, hs,
+                                             kv_mul, M, pos0)))
+                return r;
+            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_att, dim, M, &L.wq_o, dim, dim, 1))) return r;
+            if ((r = awq_launch_rmsnorm_rows(ctx, t->pf_xb, t->pf_x, L.rms_ffn_weight, dim, M))) return r;
+            if ((r = awq_launch_gemm_ffn(ctx, t->pf_hb, t->pf_xb, dim, M, &L.wq_gate, &L.wq_up, dim, hidden))) return r;
+            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_hb, hidden, M, &L.wq_down, hidden, dim, 1))) return r;
+        }
+        if (done + M == n_tokens) {
+            // last token: final norm, classifier and the greedy sampler exactly as the decode path does them
+            if ((r = awq_launch_copy_row(ctx, t->s.x, t->pf_x + (size_t)(M - 1) * dim, dim))) return r;
+            if ((r = awq_launch_set_pos(ctx, t->s.pos, t->s.shared_pos, pos_start + n_tokens - 1))) return r;
+            if ((r = awq_launch_matvec_f16(ctx, t->s.logits, t->s.x, t->wcls, dim, p.vocab_size, t->rms_final, nullptr))) return r;
+            if ((r = awq_launch_argmax(ctx, t->s.logits, p.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token,
+                                       t->tokens_dev)))
+                return r;
+        }
+    }
+    return AWQ_OK;
+}
+
 int awq_transformer_trace(awq_transformer* t, int enable, long long* host_out, int max_entries, int* nphases) {
     AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
     if (int r = awq_bind(t->ctx)) return r;
@@ -654,6 +742,8 @@ int awq_transformer_trace(awq_transformer* t, int enable, long long* host_out, i
         AWQ_HIP_TRY(hipStreamSynchronize(t->ctx->stream));
         AWQ_HIP_TRY(hipFree(t->tk_trace));
         t->tk_trace = nullptr;
+    t->pf_rows = 0;
+    t->pf_x = t->pf_xb = t->pf_q = t->pf_att = t->pf_hb = nullptr;
     }
     return AWQ_OK;
 }

@@ -70,6 +70,10 @@ class Transformer:
     def forward(self, gen_token=True, use_graph=False, mode=SCHEDULE_FUSED):
         check(lib.awq_transformer_forward(self.h, int(gen_token), int(use_graph), mode))
 
+    def prefill(self, n_tokens, gen_token=True):
+        """Consume n_tokens prompt tokens (already in the token list, from the current position) in one batched pass."""
+        check(lib.awq_transformer_prefill(self.h, n_tokens, int(gen_token)))
+
     def generate(self, prompt_tokens, steps, ignore_eos=False, use_graph=False, mode=SCHEDULE_FUSED, on_logits=None):
         """The loop of generate_thread (llama2_q4.cu:697-745) without text output.
 

@@ -184,3 +184,8 @@ def argmax_advance(ctx, logits, size, tokens, pos_host, pos_dev, write_token):
 def dequant(ctx, out, w, K, N):
     """(q - z) * scale materialised in fp16 (gpu_kernels.h:204-205)."""
     check(lib.awq_dequant(ctx.h, _addr(out), C.byref(w.c), K, N))
+
+
+def gemm_q(ctx, out, ldo, a, lda, M, w, K, N, accum=False):
+    """Batched form of matmul(QWeight) for M activation rows (prefill); no launcher of this kind exists in the reference."""
+    check(lib.awq_gemm_int4(ctx.h, _addr(out), ldo, _addr(a), lda, M, C.byref(w.c), K, N, int(accum)))

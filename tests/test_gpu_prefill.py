@@ -1,0 +1,100 @@
+"""GPU parity of the multi-token prefill path: the int4 x fp16 MFMA GEMM against fp64, and a whole prefill against
+the oracle's token-by-token run (KV cache contents and last-token logits within rel-L2 1e-2, same next token)."""
+import numpy as np
+import pytest
+
+import llama_cu_awq_amd as A
+from llama_cu_awq_amd import synth
+from oracle import oracle
+from tests.helpers import f16, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("M,K,N", [(128, 128, 128), (1, 256, 128), (37, 512, 256), (512, 4096, 256), (200, 11008, 128), (130, 1024, 384)])
+def test_gemm_int4_vs_fp64(ctx, M, K, N):
+    key = synth.stream_key(30, M, K, N)
+    w, z, s = synth.make_qweight(key, K, N)
+    a = synth.normal_f16(synth.stream_key(key, "a"), M * K)
+    qw = A.QWeight.upload(ctx, w, z, s)
+    dout = ctx.zeros(M * N * 2)
+    A.gemm_q(ctx, dout, N, ctx.upload(a), K, M, qw, K, N)
+    got = f16(dout.download(np.uint16)).reshape(M, N)
+    # truth: the dequantised fp16 weights (bit-exact definition) times the activations in fp64
+    w16 = synth.dequantize(w, z, s, K).astype(np.float32).astype(np.float16).astype(np.float64)
+    truth = a.astype(np.float64).reshape(M, K) @ w16.T
+    assert rel_l2(got, truth) <= 1e-3
+    # residual epilogue
+    resid = synth.normal_f16(synth.stream_key(key, "r"), M * N)
+    dout = ctx.upload(resid)
+    A.gemm_q(ctx, dout, N, ctx.upload(a), K, M, qw, K, N, accum=True)
+    got = f16(dout.download(np.uint16)).reshape(M, N)
+    assert rel_l2(got, truth + resid.astype(np.float64).reshape(M, N)) <= 1e-3
+
+
+def test_gemm_shape_guard(ctx):
+    buf = ctx.alloc(1 << 16)
+    qw = A.QWeight(buf, buf, buf)
+    for M, K, N in ((4, 48, 128), (4, 64, 64), (0, 64, 128)):
+        with pytest.raises(A.AwqError) as e:
+            A.gemm_q(ctx, buf, N, buf, K, M, qw, K, N)
+        assert e.value.code == -2
+
+
+CFG = dict(dim=512, hidden_dim=1536, n_layers=3, n_heads=4, n_kv_heads=4, vocab_size=1024, seq_len=192, rope_theta=10000.0)
+CFG_GQA = dict(dim=512, hidden_dim=1280, n_layers=2, n_heads=8, n_kv_heads=2, vocab_size=512, seq_len=96, rope_theta=10000.0)
+
+
+@pytest.mark.parametrize("cfg,n_prompt", [(CFG, 130), (CFG, 16), (CFG, 1), (CFG_GQA, 70)])
+def test_prefill_matches_token_by_token_oracle(ctx, cfg, n_prompt):
+    img = synth.make_model_image(cfg, seed=31)
+    t = A.Transformer(ctx, image=img)
+    o = oracle.Model(img)
+    prompt = synth.prompt_tokens(31, n_prompt, cfg["vocab_size"])
+    o.reset(prompt)
+    for i in range(n_prompt):
+        o.forward(i >= n_prompt - 1)
+    t.reset(prompt)
+    t.prefill(n_prompt, gen_token=True)
+    ctx.sync()
+    assert t.pos == n_prompt
+    kv_dim = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"]
+    n_layers, seq = cfg["n_layers"], cfg["seq_len"]
+    for name in ("key_cache", "value_cache"):
+        got = f16(t.download(name, n_layers * seq * kv_dim)).reshape(n_layers, seq, kv_dim)[:, :n_prompt]
+        want = f16(o.buffer(name, n_layers * seq * kv_dim)).reshape(n_layers, seq, kv_dim)[:, :n_prompt]
+        assert rel_l2(got, want) <= 1e-2, name
+        for l in range(n_layers):
+            assert rel_l2(got[l], want[l]) <= 1e-2, (name, l)
+    got_logits = f16(t.download("logits", cfg["vocab_size"]))
+    want_logits = f16(o.buffer("logits", cfg["vocab_size"]))
+    assert rel_l2(got_logits, want_logits) <= 1e-2
+    assert t.token(n_prompt) == o.tokens(n_prompt + 1)[n_prompt]
+    # decoding continues from the prefilled state and keeps matching the oracle
+    for i in range(8):
+        ctx.sync()
+        t.forward(True, False, A.SCHEDULE_FUSED)
+        o.forward(True)
+    ctx.sync()
+    assert [t.token(i) for i in range(n_prompt + 9)] == o.tokens(n_prompt + 9)
+    t.close()
+    o.close()
+
+
+def test_prefill_in_two_parts_equals_one(ctx):
+    """A prompt consumed as prefill(40) + prefill(30) leaves the same state as prefill(70)."""
+    img = synth.make_model_image(CFG, seed=32)
+    prompt = synth.prompt_tokens(32, 70, CFG["vocab_size"])
+    kv = CFG["n_layers"] * CFG["seq_len"] * CFG["dim"]
+    states = []
+    for parts in ((70,), (40, 30)):
+        t = A.Transformer(ctx, image=img)
+        t.reset(prompt)
+        for i, n in enumerate(parts):
+            t.prefill(n, gen_token=(i == len(parts) - 1))
+        ctx.sync()
+        states.append((t.download("key_cache", kv), t.download("value_cache", kv), t.download("logits", CFG["vocab_size"]), t.pos, t.token(70)))
+        t.close()
+    a, b = states
+    assert a[3] == b[3] == 70 and a[4] == b[4]
+    assert rel_l2(f16(a[0]), f16(b[0])) <= 1e-3 and rel_l2(f16(a[1]), f16(b[1])) <= 1e-3 and rel_l2(f16(a[2]), f16(b[2])) <= 2e-3
