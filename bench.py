@@ -45,6 +45,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=12, help="tokens of the same model timed on the CPU oracle (0 = skip)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--prefill", type=int, default=512, help="also time a batched prefill of this many prompt tokens (0 = skip)")
     ap.add_argument("--only-kernels", action="store_true", help="skip the decode loop: run only the per-kernel loops and a 256 MiB device copy (for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -162,6 +163,33 @@ def main():
     gemv_bytes = qweight_bytes(dim, dim) + 4 * dim
     gemv_gbps = gemv_bytes / gemv_us / 1e3
 
+    # ---- prefill (7B shape, M prompt tokens in one batched pass on the matrix cores)
+    prefill = None
+    if args.prefill > 0 and not args.only_kernels and args.prefill <= cfg["seq_len"]:
+        M = args.prefill
+        ptoks = synth.prompt_tokens(args.seed + 1, M, vocab)
+        times = []
+        for rep in range(3):
+            model.reset(ptoks)
+            ctx.sync()
+            ctx.record(ev0)
+            model.prefill(M, gen_token=True)
+            ctx.record(ev1)
+            ctx.sync()
+            times.append(ctx.elapsed_ms(ev0, ev1))
+        pf_ms = min(times[1:])
+        L, V = cfg["n_layers"], vocab
+        proj_flops = 2.0 * M * L * (2 * dim * dim + 2 * dim * kv_dim + 3 * dim * hid) + 2.0 * dim * V
+        attn_flops = 2.0 * 2 * L * cfg["n_heads"] * (dim // cfg["n_heads"]) * (M * (M + 1) / 2)
+        prefill = {
+            "tokens": M,
+            "ms": round(pf_ms, 3),
+            "tok_per_s": round(M / pf_ms * 1e3, 1),
+            "tflops": round((proj_flops + attn_flops) / pf_ms / 1e9, 1),
+            "mfma_frac_of_2.5PFLOPs": round((proj_flops + attn_flops) / (pf_ms * 1e-3) / 2.5e15, 4),
+            "next_token": model.token(M),
+        }
+
     # ---- CPU baseline: the oracle on the same model, a bounded number of tokens
     cpu = None
     if args.cpu_tokens > 0:
@@ -214,6 +242,7 @@ def main():
             "us_per_launch": round(ffn_us, 3),
         },
         "cpu_baseline": cpu,
+        "prefill": prefill,
         "decode": {
             "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
             "weight_bytes_per_token": wbytes,

@@ -50,6 +50,10 @@ typedef struct awq_transformer awq_transformer; /* weights + run state of one mo
 /* Text of the most recent error recorded by any call in this process. */
 const char* awq_last_error(void);
 
+/* ---- device enumeration: get_and_print_gpu_info(), llama2_q4.cu:817-837 (cudaGetDeviceCount/Properties). */
+int awq_device_count(int* count);
+int awq_device_info(int device, char* name, size_t name_bytes, size_t* global_mem_bytes, int* compute_units);
+
 /* ---- context: cudaSetDevice + cudaStreamCreate (llama2_q4.cu:685, 695) and the
  *      global `streams[rank]` (llama2_q4.cu:338-345). */
 int awq_ctx_create(int device, awq_ctx** out);
@@ -190,6 +194,13 @@ int awq_transformer_set_pos(awq_transformer* t, int pos, int token);
 #define AWQ_SCHEDULE_FUSED 1
 #define AWQ_SCHEDULE_PERSISTENT 2
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode);
+
+/* run_llama_network() alone (llama2_q4.cu:430-538): the token's logits without any sampler, for callers that sample
+ * on their own (the non-greedy branch of sample(), sampler.h:85-115).  mode: REFERENCE or FUSED; launched eagerly. */
+int awq_transformer_forward_logits(awq_transformer* t, int use_graph, int mode);
+/* The tail of the reference's samplers (gpu_kernels.h:490-500, 582-591) for a token chosen by the caller:
+ * p = pos + 1; if write_token, tokens[p] = token; pos = p (pinned-host and device copies). */
+int awq_transformer_accept(awq_transformer* t, int token, int write_token);
 
 /* ---- multi-token prefill.  No counterpart in the reference, which consumes the prompt one token per forward pass
  * (llama2_q4.cu:716-735); the contract is the state that loop would leave. ---- */

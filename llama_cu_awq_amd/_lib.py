@@ -40,6 +40,8 @@ _pq = C.POINTER(QWeightC)
 
 # name -> argtypes; every function returns int except the two noted below
 PROTOTYPES = {
+    "awq_device_count": [C.POINTER(C.c_int)],
+    "awq_device_info": [_i, C.c_char_p, _sz, C.POINTER(C.c_size_t), C.POINTER(C.c_int)],
     "awq_ctx_create": [_i, _pvp],
     "awq_ctx_create_on_stream": [_i, _vp, _pvp],
     "awq_ctx_destroy": [_vp],
@@ -79,6 +81,8 @@ PROTOTYPES = {
     "awq_transformer_forward": [_vp, _i, _i, _i],
     "awq_gemm_int4": [_vp, _vp, _i, _vp, _i, _i, _pq, _i, _i, _i],
     "awq_transformer_prefill": [_vp, _i, _i],
+    "awq_transformer_forward_logits": [_vp, _i, _i],
+    "awq_transformer_accept": [_vp, _i, _i],
     "awq_transformer_trace": [_vp, _i, C.POINTER(C.c_longlong), _i, C.POINTER(C.c_int)],
 }
 NON_STATUS = {"awq_last_error": ([], C.c_char_p), "awq_ctx_stream": ([_vp], _vp)}

@@ -23,6 +23,34 @@ extern "C" {
 
 const char* awq_last_error(void) { return g_err; }
 
+int awq_device_count(int* count) {
+    AWQ_REQUIRE(count, AWQ_ERR_ARG, "null count");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e == hipErrorNoDevice) {
+        *count = 0;
+        return AWQ_OK;
+    }
+    if (e != hipSuccess) {
+        awq_set_error("hipGetDeviceCount failed: %s", hipGetErrorString(e));
+        return AWQ_ERR_HIP;
+    }
+    *count = n;
+    return AWQ_OK;
+}
+
+int awq_device_info(int device, char* name, size_t name_bytes, size_t* global_mem_bytes, int* compute_units) {
+    hipDeviceProp_t prop;
+    AWQ_HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (name && name_bytes) {
+        strncpy(name, prop.name, name_bytes - 1);
+        name[name_bytes - 1] = 0;
+    }
+    if (global_mem_bytes) *global_mem_bytes = prop.totalGlobalMem;
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    return AWQ_OK;
+}
+
 static int ctx_init(int device, hipStream_t stream, bool owns, awq_ctx** out) {
     awq_ctx* c = new awq_ctx();
     c->device = device;

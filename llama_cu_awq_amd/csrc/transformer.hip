@@ -43,6 +43,18 @@ int awq_launch_copy_row(awq_ctx* ctx, uint16_t* dst, const uint16_t* src, int n)
 
 namespace {
 
+// p = *pos + 1; if (write_token) tokens[p] = token; *pos_host = *pos_dev = p  (the tail of the reference's samplers,
+// gpu_kernels.h:490-500 and :582-591, for a token chosen on the host)
+__global__ void accept_kernel(int token, int* tokens_host, int* tokens_dev, volatile int* pos_host, int* pos_dev, int write_token) {
+    const int p = *pos_dev + 1;
+    if (write_token) {
+        tokens_host[p] = token;
+        tokens_dev[p] = token;
+    }
+    *pos_host = p;
+    *pos_dev = p;
+}
+
 constexpr int kMaxSeqLen = 128 * 1024;  // SharedData.tokens capacity, common.h:13
 constexpr int kMaxGraphs = 8;           // llama2_q4.cu:337
 
@@ -746,6 +758,29 @@ int awq_transformer_trace(awq_transformer* t, int enable, long long* host_out, i
     t->pf_x = t->pf_xb = t->pf_q = t->pf_att = t->pf_hb = nullptr;
     }
     return AWQ_OK;
+}
+
+int awq_transformer_forward_logits(awq_transformer* t, int use_graph, int mode) {
+    AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
+    AWQ_REQUIRE(mode == AWQ_SCHEDULE_REFERENCE || mode == AWQ_SCHEDULE_FUSED, AWQ_ERR_ARG,
+                "forward_logits runs the reference or the fused schedule");
+    (void)use_graph;  // the recorded sequences include the sampler; this entry point always launches eagerly
+    awq_ctx* ctx = t->ctx;
+    if (int r = awq_bind(ctx)) return r;
+    const int seq_len = t->shared->pos + 1;
+    AWQ_REQUIRE(seq_len <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+    return network(t, seq_len, mode);
+}
+
+int awq_transformer_accept(awq_transformer* t, int token, int write_token) {
+    AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
+    AWQ_REQUIRE(token >= 0 && token < t->cfg.vocab_size, AWQ_ERR_ARG, "token out of range");
+    awq_ctx* ctx = t->ctx;
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(t->shared->pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+    hipLaunchKernelGGL(accept_kernel, dim3(1), dim3(1), 0, ctx->stream, token, t->s.shared_tokens, t->tokens_dev, t->s.shared_pos,
+                       t->s.pos, write_token);
+    return awq_check_launch("accept");
 }
 
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode) {
