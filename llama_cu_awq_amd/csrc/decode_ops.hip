@@ -6,6 +6,8 @@
 
 namespace {
 
+constexpr int kAttnFusedMaxSeq = 512;  // up to this launch size attention runs as one workgroup per head
+
 // ------------------------------------------------------------------ embed
 __global__ __launch_bounds__(256) void embed_kernel(uint16_t* x, const uint16_t* table, int dim, const int* tokens,
                                                     const int* pPos) {
@@ -161,15 +163,27 @@ __global__ __launch_bounds__(256) void attn_softmax_pv_kernel(uint16_t* output, 
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.0f;
-    for (int t = tb + wave * PW + pr; t < te; t += 4 * PW) {
-        const u32x4 v = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
-        const float e = expf(half_bits_to_float(a[t]) - m);
-        const float p = half_bits_to_float(float_to_half_bits(e / sum));  // probability rounded to fp16
+    // four rows per lane are requested before any is used (each is an HBM/L2 round trip)
+    for (int t0 = tb + wave * PW + pr; t0 - pr - wave * PW < te; t0 += 16 * PW) {
+        u32x4 vv[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const h16x2 hv = as_h2(v[i]);
-            acc[2 * i] = fmaf((float)hv[0], p, acc[2 * i]);
-            acc[2 * i + 1] = fmaf((float)hv[1], p, acc[2 * i + 1]);
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * 4 * PW;
+            if (t < te) vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * 4 * PW;
+            if (t < te) {
+                const float e = expf(half_bits_to_float(a[t]) - m);
+                const float p = half_bits_to_float(float_to_half_bits(e / sum));  // probability rounded to fp16
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const h16x2 hv = as_h2(vv[k][i]);
+                    acc[2 * i] = fmaf((float)hv[0], p, acc[2 * i]);
+                    acc[2 * i + 1] = fmaf((float)hv[1], p, acc[2 * i + 1]);
+                }
+            }
         }
     }
     // combine the PW position groups of the wave, then the 4 waves
@@ -204,6 +218,110 @@ __global__ __launch_bounds__(256) void attn_softmax_pv_kernel(uint16_t* output, 
             output[(size_t)h * head_size + tid] = float_to_half_bits(s);
         }
         if (tid == 0) counter[h] = 0;  // ready for the next launch
+    }
+}
+
+// Short contexts: one workgroup of 16 waves per head does scores, softmax and P.V in a single launch (the work is
+// a few hundred KB per head, so the launch count matters more than the parallelism).  Same arithmetic and
+// rounding points as the two-pass kernels above; the fp16 scores are also left in att.
+template <int LP>
+__global__ __launch_bounds__(1024) void attn_fused_kernel(uint16_t* output, uint16_t* att, const uint16_t* q,
+                                                          const uint16_t* key_cache, const uint16_t* value_cache, int head_size,
+                                                          int kv_mul, int row_stride, float alpha, const int* pPos) {
+    extern __shared__ float fsm[];
+    float* sc = fsm;                // [size] scores (fp16-rounded values)
+    __shared__ float red[32];
+    const int size = *pPos + 1;
+    float* acc_lds = fsm + ((size + 3) & ~3);  // [16][head_size]
+    const int h = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int PW = 64 / LP;
+    const int j = lane % LP, pr = lane / LP;
+    const int tstep = 16 * PW;  // positions covered by the workgroup per round
+    const int tfirst = wave * PW + pr;
+    const u32x4 qv = *reinterpret_cast<const u32x4*>(q + (size_t)h * head_size + j * 8);
+    const uint16_t* kh = key_cache + (size_t)(h / kv_mul) * head_size + j * 8;
+    const uint16_t* vh = value_cache + (size_t)(h / kv_mul) * head_size + j * 8;
+    uint16_t* a = att + (size_t)h * size;
+    for (int t0 = tfirst; t0 - tfirst < size; t0 += 4 * tstep) {
+        u32x4 kv[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * tstep;
+            if (t < size) kv[k] = *reinterpret_cast<const u32x4*>(kh + (size_t)t * row_stride);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * tstep;
+            float s = 0.0f;
+            if (t < size) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) s = dot2(kv[k][i], qv[i], s);
+            }
+            s = group_sum<LP>(s);
+            if (j == 0 && t < size) {
+                const uint16_t hb = float_to_half_bits(s * alpha);
+                a[t] = hb;
+                sc[t] = half_bits_to_float(hb);
+            }
+        }
+    }
+    __syncthreads();
+    float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed
+    for (int t = tid; t < size; t += 1024) m = fmaxf(m, sc[t]);
+    m = wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = red[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) m = fmaxf(m, red[w]);
+    float sum = 0.0f;
+    for (int t = tid; t < size; t += 1024) sum += expf(sc[t] - m);
+    sum = wave_sum(sum);
+    if (lane == 0) red[16 + wave] = sum;
+    __syncthreads();
+    sum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 16; w++) sum += red[16 + w];
+
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.0f;
+    for (int t0 = tfirst; t0 - tfirst < size; t0 += 4 * tstep) {
+        u32x4 vv[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * tstep;
+            if (t < size) vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * tstep;
+            if (t < size) {
+                const float e = expf(sc[t] - m);
+                const float pv = half_bits_to_float(float_to_half_bits(e / sum));
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const h16x2 hv = as_h2(vv[k][i]);
+                    acc[2 * i] = fmaf((float)hv[0], pv, acc[2 * i]);
+                    acc[2 * i + 1] = fmaf((float)hv[1], pv, acc[2 * i + 1]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        for (int off = LP; off < 64; off <<= 1) acc[i] += __shfl_xor(acc[i], off);
+    if (pr == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc_lds[wave * head_size + j * 8 + i] = acc[i];
+    }
+    __syncthreads();
+    if (tid < head_size) {
+        float total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 16; w++) total += acc_lds[w * head_size + tid];
+        output[(size_t)h * head_size + tid] = float_to_half_bits(total);
     }
 }
 
@@ -367,6 +485,12 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
                      const int* pos) {
     const int row_stride = num_heads * head_size / kv_mul;
     const float alpha = (float)(1.0 / sqrt((double)head_size));
+    if (max_seq_len <= kAttnFusedMaxSeq) {
+        const size_t lds = (size_t)(((max_seq_len + 3) & ~3) + 16 * head_size) * sizeof(float);
+        hipLaunchKernelGGL((attn_fused_kernel<LP>), dim3(num_heads), dim3(1024), lds, ctx->stream, output, att, q, key_cache,
+                           value_cache, head_size, kv_mul, row_stride, alpha, pos);
+        return awq_check_launch("attn_fused");
+    }
     hipLaunchKernelGGL((attn_scores_kernel<LP>), dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, ctx->stream, att, q,
                        key_cache, head_size, kv_mul, row_stride, alpha, pos);
     if (int r = awq_check_launch("attn_scores")) return r;

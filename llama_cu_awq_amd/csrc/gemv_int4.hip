@@ -17,6 +17,8 @@
 // OR-ing them into the mantissa of 1024.0, products are accumulated in fp32 by
 // v_dot2_f32_f16 with the 1024 offset and the zero point cancelled through
 // per-chunk constants, and the group scale is applied once per 32 elements.
+#include <stdlib.h>
+
 #include "common.hpp"
 
 namespace {
@@ -40,6 +42,9 @@ struct GemvParams {
     float inv_gpu_count;
     int loff[3];             // -1: none; else out += loff + *pos * N
     const int* pos;
+    int groups_per_wg;       // row groups (4 waves x R rows) a workgroup walks through
+    const float2* rope;      // fused RoPE: (cos, sin) table [position][head_size/2], or null
+    int head_size;           // for the fused RoPE row pairing
 };
 
 enum { KIND_SINGLE = 0, KIND_QKV = 1, KIND_FFN = 2 };
@@ -187,7 +192,17 @@ __device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const GemvParams&
     __syncthreads();
 }
 
-template <int R, int KIND, bool NORM>
+// Logical index li of a workgroup's row space -> matrix row.  With ROPE, consecutive indices (2j, 2j+1) are the two
+// rows (i, i + head/2) of one rotation pair, so that one wave holds both.
+template <bool ROPE>
+__device__ __forceinline__ int map_row(int li, int head_size) {
+    if (!ROPE) return li;
+    const int half = head_size >> 1;
+    const int pi = li >> 1;
+    return (pi / half) * head_size + (pi % half) + (li & 1) * half;
+}
+
+template <int R, int KIND, bool NORM, bool ROPE>
 __global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
     extern __shared__ u32x4 xs[];
     __shared__ float red[4];
@@ -195,75 +210,136 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
     const int wave = threadIdx.x >> 6;
     const int C = p.C;
     const int pwh = C * 4;
+    const int P = (C + 63) >> 6;  // 64-lane passes per row
     float2* ab = reinterpret_cast<float2*>(xs + 4 * C);
     const int which = (KIND == KIND_QKV) ? blockIdx.y : 0;
-    const int row0 = min((blockIdx.x * 4 + wave) * R, p.N - 1);  // a wave past N recomputes the last row, stores nothing
+    const bool rope_here = ROPE && which != 2;
     uint32_t magic = 0x64006400u;  // fp16 pair (1024.0, 1024.0), kept in a VGPR
     asm("" : "+v"(magic));
 
     constexpr int NS = (KIND == KIND_FFN) ? 2 * R : R;
+    const Int4Mat m0 = (KIND == KIND_QKV) ? (which == 0 ? p.m[0] : (which == 1 ? p.m[1] : p.m[2])) : p.m[0];
+    const Int4Mat m1 = p.m[1];  // FFN: up
+
+    // this workgroup's row groups
+    const int groups_total = (p.N + 4 * R - 1) / (4 * R);
+    const int g_begin = blockIdx.x * p.groups_per_wg;
+    const int g_end = min(groups_total, g_begin + p.groups_per_wg);
+    const int total = (g_end - g_begin) * P;  // stages this wave walks through
+
+    // ---- load cursor
     const uint32_t* wrow[NS];
     const uint32_t* zrow[NS];
     const uint16_t* srow[NS];
+    int lg = g_begin, lp = 0, lit = 0;
+    auto set_rows = [&](int g) {
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        const int row = min(row0 + r, p.N - 1);  // rows past N are recomputed and not stored
-        if (KIND == KIND_FFN) {
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                wrow[2 * r + j] = p.m[j].w + (size_t)row * pwh;
-                zrow[2 * r + j] = p.m[j].z + (size_t)row * p.pzh;
-                srow[2 * r + j] = p.m[j].s + (size_t)row * p.sh;
+        for (int r = 0; r < R; r++) {
+            const int li = min((g * 4 + wave) * R + r, p.N - 1);  // indices past N are recomputed, never stored
+            const int row = rope_here ? map_row<true>(li, p.head_size) : li;
+            if (KIND == KIND_FFN) {
+                wrow[2 * r] = m0.w + (size_t)row * pwh;
+                zrow[2 * r] = m0.z + (size_t)row * p.pzh;
+                srow[2 * r] = m0.s + (size_t)row * p.sh;
+                wrow[2 * r + 1] = m1.w + (size_t)row * pwh;
+                zrow[2 * r + 1] = m1.z + (size_t)row * p.pzh;
+                srow[2 * r + 1] = m1.s + (size_t)row * p.sh;
+            } else {
+                wrow[r] = m0.w + (size_t)row * pwh;
+                zrow[r] = m0.z + (size_t)row * p.pzh;
+                srow[r] = m0.s + (size_t)row * p.sh;
             }
-        } else {
-            const Int4Mat m = (KIND == KIND_QKV) ? (which == 0 ? p.m[0] : (which == 1 ? p.m[1] : p.m[2])) : p.m[0];
-            wrow[r] = m.w + (size_t)row * pwh;
-            zrow[r] = m.z + (size_t)row * p.pzh;
-            srow[r] = m.s + (size_t)row * p.sh;
         }
-    }
+    };
+    auto load_next = [&](Stage<NS>& st) {
+        if (lit < total) {
+            load_stage<NS>(st, wrow, zrow, srow, lp * 64 + lane, C);
+            lit++;
+            lp++;
+            if (lp == P) {
+                lp = 0;
+                lg++;
+                if (lit < total) set_rows(lg);
+            }
+        }
+    };
 
     float sum[NS];
 #pragma unroll
     for (int i = 0; i < NS; i++) sum[i] = 0.0f;
 
-    // The first two passes of packed weights are requested before x is staged, so
-    // that their HBM latency overlaps the staging (and the RMSNorm reduction).
-    Stage<NS> a, b;
-    load_stage<NS>(a, wrow, zrow, srow, lane, C);
-    load_stage<NS>(b, wrow, zrow, srow, lane + 64, C);
-    stage_x<NORM>(xs, ab, p, red);
-    for (int c = lane; c < C + lane; c += 128) {  // wave-uniform trip count
-        const int c1 = c + 64;
-        consume_stage<NS>(a, xs, ab, c, C, sum, magic);
-        load_stage<NS>(a, wrow, zrow, srow, c1 + 64, C);
-        consume_stage<NS>(b, xs, ab, c1, C, sum, magic);
-        load_stage<NS>(b, wrow, zrow, srow, c1 + 128, C);
-    }
-
+    // ---- consume cursor
+    int cg = g_begin, cp = 0;
+    auto finish_group = [&]() {
 #pragma unroll
-    for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]);
-
-    if (lane == 0 && (blockIdx.x * 4 + wave) * R < p.N) {
-        uint16_t* out = (KIND == KIND_QKV) ? (which == 0 ? p.out[0] : (which == 1 ? p.out[1] : p.out[2])) : p.out[0];
-        const int loff = (KIND == KIND_QKV) ? (which == 0 ? p.loff[0] : (which == 1 ? p.loff[1] : p.loff[2])) : p.loff[0];
-        if (loff != -1) out += (size_t)loff + (size_t)(*p.pos) * p.N;
+        for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]);
+        const int li0 = (cg * 4 + wave) * R;
+        if (lane == 0 && li0 < p.N) {
+            uint16_t* out = (KIND == KIND_QKV) ? (which == 0 ? p.out[0] : (which == 1 ? p.out[1] : p.out[2])) : p.out[0];
+            const int loff = (KIND == KIND_QKV) ? (which == 0 ? p.loff[0] : (which == 1 ? p.loff[1] : p.loff[2])) : p.loff[0];
+            if (loff != -1) out += (size_t)loff + (size_t)(*p.pos) * p.N;
+            if (rope_here) {
+                // q/k are rounded to fp16 and then rotated, as the separate RoPE kernel does (gpu_kernels.h:351-361)
+                const int half = p.head_size >> 1;
+                const float2* cs = p.rope + (size_t)(*p.pos) * half;
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const int row = row0 + r;
-            if (row < p.N) {
-                float v;
-                if (KIND == KIND_FFN) {
-                    // gate = stream 2r, up = stream 2r+1 (gpu_kernels.h:276-281)
-                    float g = sum[2 * r];
-                    g *= 1.0f / (1.0f + expf(-g));
-                    v = g * sum[2 * r + 1];
-                } else {
-                    v = sum[r];
-                    if (KIND == KIND_SINGLE && p.accum) v += half_bits_to_float(out[row]) * p.inv_gpu_count;
+                for (int r = 0; r < R; r += 2) {
+                    const int li = li0 + r;
+                    if (li < p.N) {
+                        const int row = map_row<true>(li, p.head_size);
+                        const float v0 = half_bits_to_float(float_to_half_bits(sum[r]));
+                        const float v1 = half_bits_to_float(float_to_half_bits(sum[r + 1]));
+                        const float2 c = cs[row % half];
+                        out[row] = float_to_half_bits(v0 * c.x - v1 * c.y);
+                        out[row + half] = float_to_half_bits(v0 * c.y + v1 * c.x);
+                    }
                 }
-                out[row] = float_to_half_bits(v);
+            } else {
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const int row = li0 + r;
+                    if (row < p.N) {
+                        float v;
+                        if (KIND == KIND_FFN) {
+                            // gate = stream 2r, up = stream 2r+1 (gpu_kernels.h:276-281)
+                            float g = sum[2 * r];
+                            g *= 1.0f / (1.0f + expf(-g));
+                            v = g * sum[2 * r + 1];
+                        } else {
+                            v = sum[r];
+                            if (KIND == KIND_SINGLE && p.accum) v += half_bits_to_float(out[row]) * p.inv_gpu_count;
+                        }
+                        out[row] = float_to_half_bits(v);
+                    }
+                }
             }
+        }
+#pragma unroll
+        for (int i = 0; i < NS; i++) sum[i] = 0.0f;
+    };
+    auto consume = [&](const Stage<NS>& st) {
+        consume_stage<NS>(st, xs, ab, cp * 64 + lane, C, sum, magic);
+        cp++;
+        if (cp == P) {
+            finish_group();
+            cp = 0;
+            cg++;
+        }
+    };
+
+    // The first two stages of packed weights are requested before x is staged, so that their HBM latency overlaps
+    // the staging (and the RMSNorm reduction); after that two stages stay in flight across row groups.
+    Stage<NS> a, b;
+    if (total > 0) set_rows(lg);
+    load_next(a);
+    load_next(b);
+    stage_x<NORM>(xs, ab, p, red);
+    for (int it = 0; it < total; it += 2) {
+        consume(a);
+        load_next(a);
+        if (it + 1 < total) {
+            consume(b);
+            load_next(b);
         }
     }
 }
@@ -316,20 +392,39 @@ void fill_common(GemvParams& p, const uint16_t* x, int K, int N) {
     p.inv_gpu_count = 1.0f;
     p.loff[0] = p.loff[1] = p.loff[2] = -1;
     p.pos = nullptr;
+    p.groups_per_wg = 1;
+    p.rope = nullptr;
+    p.head_size = 0;
 }
 
 Int4Mat to_mat(const awq_qweight* w) { return Int4Mat{w->weight, w->zeros, w->scales}; }
 
 bool qw_ok(const awq_qweight* w) { return w && w->weight && w->zeros && w->scales; }
 
-template <int R, int KIND>
-int launch(awq_ctx* ctx, const GemvParams& p, int grid_y, const char* what) {
-    const dim3 grid(div_up(p.N, 4 * R), grid_y);
+// Row groups per workgroup: enough workgroups to fill the chip several times over, but at least ~8 pipeline stages
+// per wave when the matrix is large enough to afford it (a stage = one 64-lane pass over the wave's rows).
+int pick_groups_per_wg(int groups_total, int passes) {
+    static int forced = -1;
+    if (forced < 0) {
+        const char* e = getenv("AWQ_GEMV_GROUPS_PER_WG");
+        forced = e ? atoi(e) : 0;
+    }
+    if (forced > 0) return forced;
+    int gpw = 1;
+    while (gpw * passes < 8 && groups_total / (gpw * 2) >= 512) gpw *= 2;
+    return gpw;
+}
+
+template <int R, int KIND, bool ROPE>
+int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
+    const int groups_total = div_up(p.N, 4 * R);
+    p.groups_per_wg = pick_groups_per_wg(groups_total, div_up(p.C, 64));
+    const dim3 grid(div_up(groups_total, p.groups_per_wg), grid_y);
     const size_t lds = (size_t)p.C * 72;  // activations + per-chunk constants
     if (p.norm_w)
-        hipLaunchKernelGGL((gemv_int4_kernel<R, KIND, true>), grid, dim3(256), lds, ctx->stream, p);
+        hipLaunchKernelGGL((gemv_int4_kernel<R, KIND, true, ROPE>), grid, dim3(256), lds, ctx->stream, p);
     else
-        hipLaunchKernelGGL((gemv_int4_kernel<R, KIND, false>), grid, dim3(256), lds, ctx->stream, p);
+        hipLaunchKernelGGL((gemv_int4_kernel<R, KIND, false, ROPE>), grid, dim3(256), lds, ctx->stream, p);
     return awq_check_launch(what);
 }
 
@@ -350,15 +445,17 @@ int awq_launch_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const
     p.norm_w = norm_w;
     p.norm_out = norm_out;
     // 2 rows per wave keep >= 2 workgroups per CU busy at N = 4096; 4 rows amortise staging on big N
-    if (N >= 8192) return launch<4, KIND_SINGLE>(ctx, p, 1, "gemv_int4");
-    return launch<2, KIND_SINGLE>(ctx, p, 1, "gemv_int4");
+    if (N >= 8192) return launch<4, KIND_SINGLE, false>(ctx, p, 1, "gemv_int4");
+    return launch<2, KIND_SINGLE, false>(ctx, p, 1, "gemv_int4");
 }
 
 int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
                    const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw, int K, int N, int loff,
-                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out) {
+                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out, const float2* rope, int head_size) {
     GemvParams p;
     fill_common(p, x, K, N);
+    p.rope = rope;
+    p.head_size = head_size;
     p.m[0] = to_mat(qw);
     p.m[1] = to_mat(kw);
     p.m[2] = to_mat(vw);
@@ -370,7 +467,8 @@ int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* val
     p.pos = pos;
     p.norm_w = norm_w;
     p.norm_out = norm_out;
-    return launch<4, KIND_QKV>(ctx, p, 3, "qkv_matvec");
+    if (rope) return launch<4, KIND_QKV, true>(ctx, p, 3, "qkv_matvec_rope");
+    return launch<4, KIND_QKV, false>(ctx, p, 3, "qkv_matvec");
 }
 
 int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w, const awq_qweight* up_w, int K,
@@ -382,7 +480,7 @@ int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qwe
     p.out[0] = out;
     p.norm_w = norm_w;
     p.norm_out = norm_out;
-    return launch<2, KIND_FFN>(ctx, p, 1, "ffn_matvec_silu");
+    return launch<2, KIND_FFN, false>(ctx, p, 1, "ffn_matvec_silu");
 }
 
 extern "C" {
@@ -404,7 +502,7 @@ int awq_qkv_matvec(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* val
     if (int r = check_shape(K, N)) return r;
     AWQ_REQUIRE(q && key_cache && value_cache && x && qw_ok(qw) && qw_ok(kw) && qw_ok(vw), AWQ_ERR_ARG, "null pointer");
     AWQ_REQUIRE(loff >= 0 && pos, AWQ_ERR_ARG, "qkv needs loff >= 0 and a position pointer");
-    return awq_launch_qkv(ctx, q, key_cache, value_cache, x, qw, kw, vw, K, N, loff, pos, nullptr, nullptr);
+    return awq_launch_qkv(ctx, q, key_cache, value_cache, x, qw, kw, vw, K, N, loff, pos, nullptr, nullptr, nullptr, 0);
 }
 
 int awq_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w, const awq_qweight* up_w,

@@ -18,7 +18,7 @@ int awq_launch_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const
                            int gpu_count, int loff, const int* pos, const uint16_t* norm_w, uint16_t* norm_out);
 int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
                    const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw, int K, int N, int loff,
-                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out);
+                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out, const float2* rope, int head_size);
 int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w, const awq_qweight* up_w, int K,
                    int N, const uint16_t* norm_w, uint16_t* norm_out);
 int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
@@ -42,6 +42,17 @@ int awq_launch_set_pos(awq_ctx* ctx, int* pos_dev, volatile int* pos_host, int v
 int awq_launch_copy_row(awq_ctx* ctx, uint16_t* dst, const uint16_t* src, int n);
 
 namespace {
+
+// (cos, sin) of pos * theta^(-2i/head) for every position and pair index, with the arithmetic of the RoPE kernel
+// (gpu_kernels.h:346-350), so that the fused QKV epilogue rotates with exactly the values that kernel would compute.
+__global__ void rope_table_kernel(float2* table, int half, int head_size, float rope_theta) {
+    const int pos = blockIdx.x;
+    const int i = threadIdx.x;
+    const int head_dim = (i * 2) % head_size;
+    const float freq = 1.0f / powf(rope_theta, head_dim / (float)head_size);
+    const float val = pos * freq;
+    table[(size_t)pos * half + i] = make_float2(cosf(val), sinf(val));
+}
 
 // p = *pos + 1; if (write_token) tokens[p] = token; *pos_host = *pos_dev = p  (the tail of the reference's samplers,
 // gpu_kernels.h:490-500 and :582-591, for a token chosen on the host)
@@ -79,6 +90,7 @@ struct awq_transformer {
     hipGraphExec_t graphs[2][kMaxGraphs];
     bool captured[2][kMaxGraphs];
     int* tokens_dev;  // device mirror of SharedData.tokens (the persistent kernel reads its input token here)
+    float2* rope_table;  // [seq_len][head_size/2] (cos, sin)
     // plan of the persistent per-token kernel
     bool tk_ok;
     char tk_why[160];  // why the persistent kernel cannot run this model, when !tk_ok
@@ -183,6 +195,10 @@ int alloc_state(awq_transformer* t) {
     memset((void*)t->shared, 0, sizeof(SharedData));
     AWQ_HIP_TRY(hipMalloc((void**)&t->tokens_dev, (size_t)(c.seq_len + 8) * sizeof(int)));
     AWQ_HIP_TRY(hipMemset(t->tokens_dev, 0, (size_t)(c.seq_len + 8) * sizeof(int)));
+    const int head = c.dim / c.n_heads;
+    AWQ_HIP_TRY(hipMalloc((void**)&t->rope_table, (size_t)c.seq_len * (head / 2) * sizeof(float2)));
+    hipLaunchKernelGGL(rope_table_kernel, dim3(c.seq_len), dim3(head / 2), 0, t->ctx->stream, t->rope_table, head / 2, head, c.rope_theta);
+    if (int r = awq_check_launch("rope_table")) return r;
     s.shared_pos = &t->shared->pos;
     s.shared_tokens = t->shared->tokens;
     return AWQ_OK;
@@ -205,6 +221,7 @@ void release(awq_transformer* t) {
     (void)hipFree(t->s.pos);
     if (t->shared) (void)hipHostFree(t->shared);
     (void)hipFree(t->tokens_dev);
+    (void)hipFree(t->rope_table);
     (void)hipFree(t->tk_phases);
     (void)hipFree(t->tk_sync);
     (void)hipFree(t->tk_trace);
@@ -224,6 +241,7 @@ awq_transformer* new_transformer(awq_ctx* ctx) {
     t->blob_bytes = 0;
     t->shared = nullptr;
     t->tokens_dev = nullptr;
+    t->rope_table = nullptr;
     t->tk_ok = false;
     t->tk_why[0] = 0;
     t->tk_phases = nullptr;
@@ -460,7 +478,7 @@ int network_fused(awq_transformer* t, int seq_len_bin) {
         const int loff = l * p.seq_len * kv_dim;
         if (dim == kv_dim) {
             if ((r = awq_launch_qkv(ctx, s.q, s.key_cache, s.value_cache, s.x, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, loff, pPos,
-                                    L.rms_att_weight, nullptr)))
+                                    L.rms_att_weight, nullptr, t->rope_table, head_size)))
                 return r;
         } else {
             if ((r = awq_launch_matvec_int4(ctx, s.q, s.x, &L.wq_q, dim, dim, 0, 1, -1, nullptr, L.rms_att_weight, nullptr)))
@@ -471,8 +489,8 @@ int network_fused(awq_transformer* t, int seq_len_bin) {
             if ((r = awq_launch_matvec_int4(ctx, s.value_cache, s.x, &L.wq_v, dim, kv_dim, 0, 1, loff, pPos, L.rms_att_weight,
                                             nullptr)))
                 return r;
+            if ((r = awq_rope(ctx, s.q, s.key_cache, p.n_heads, p.n_kv_heads, head_size, pPos, loff, p.rope_theta))) return r;
         }
-        if ((r = awq_rope(ctx, s.q, s.key_cache, p.n_heads, p.n_kv_heads, head_size, pPos, loff, p.rope_theta))) return r;
         if ((r = awq_attention(ctx, s.xb, s.q, s.key_cache + loff, s.value_cache + loff, s.att, p.n_heads, head_size, kv_mul,
                                seq_len_bin, pPos)))
             return r;
