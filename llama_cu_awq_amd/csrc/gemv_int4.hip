@@ -64,7 +64,10 @@ __device__ __forceinline__ float chunk_dot(const u32x4 w, const float zf, const 
                                            const uint32_t magic) {
     float acc = fmaf(-zf, A, -B);
 #pragma unroll
-    for (int qi = 0; qi < 4; qi++) {
+#ifndef AWQ_PROBE_QI
+#define AWQ_PROBE_QI 4
+#endif
+    for (int qi = 0; qi < AWQ_PROBE_QI; qi++) {
         const uint32_t d = w[qi];
         const uint32_t d8 = d >> 8;
         acc = dot2((d & 0x000F000Fu) | magic, xq[qi][0], acc);
@@ -75,119 +78,140 @@ __device__ __forceinline__ float chunk_dot(const u32x4 w, const float zf, const 
     return acc;
 }
 
+// One 64-lane pass over the NS row streams of a wave: 16 bytes of packed weights per lane and stream, the zero-point
+// dword and the scale that cover them, and (residual form) the value the result is added to.
 template <int NS>
 struct Stage {
     u32x4 w[NS];
     uint32_t zw[NS];
     uint16_t s[NS];
+    uint16_t res[NS];
 };
 
-template <int NS>
-__device__ __forceinline__ void load_stage(Stage<NS>& st, const uint32_t* const (&wrow)[NS],
-                                           const uint32_t* const (&zrow)[NS], const uint16_t* const (&srow)[NS], int c,
-                                           int C) {
-    if (c < C) {
-#pragma unroll
-        for (int i = 0; i < NS; i++) {
-            st.w[i] = load_nt(reinterpret_cast<const u32x4*>(wrow[i]) + c);
-            st.zw[i] = zrow[i][c >> 5];
-            st.s[i] = srow[i][c >> 2];
-        }
-    }
-}
+// Staging of x (K halves) into LDS: xs[qi*C + c] holds the 8 activations of dword qi of chunk c as pairs
+// (x0,x4)(x1/16,x5/16)(x2,x6)(x3/16,x7/16), and ab[c] = {A, B} the chunk constants described at chunk_dot.  Elements
+// in [K, 32*C) are zero.  With NORM the vector is RMS-normalised on the way in with the reference's arithmetic
+// (gpu_kernels.h:72-105): o = half(x * (rsqrt(mean(x^2) + 1e-5) * w)).
+//
+// Loads return in order, so the activations are requested (load_x) before the first stages of packed weights and
+// staged (stage_x) while those are still on their way: XP pieces of 8 halves per thread travel in registers, the rest
+// of a longer vector is fetched late by stage_x itself.
+constexpr int XP = 2;
 
-template <int NS>
-__device__ __forceinline__ void consume_stage(const Stage<NS>& st, const u32x4* xs, const float2* ab, int c, int C,
-                                              float (&sum)[NS], const uint32_t magic) {
-    if (c < C) {
-        u32x4 xq[4];
-#pragma unroll
-        for (int qi = 0; qi < 4; qi++) xq[qi] = xs[qi * C + c];
-        const float2 cab = ab[c];
-        const int zshift = ((c >> 2) & 7) * 4;
-#pragma unroll
-        for (int i = 0; i < NS; i++) {
-            const float zf = (float)((st.zw[i] >> zshift) & 0xFu);
-            const float acc = chunk_dot(st.w[i], zf, xq, cab.x, cab.y, magic);
-            sum[i] = fmaf(half_bits_to_float(st.s[i]), acc, sum[i]);
-        }
-    }
-}
-
-// Stage x (K halves) into LDS: xs[qi*C + c] holds the 8 activations of dword qi
-// of chunk c as pairs (x0,x4)(x1/16,x5/16)(x2,x6)(x3/16,x7/16), and ab[c] =
-// {A, B} the chunk constants described at chunk_dot.  Elements in [K, 32*C)
-// are zero.  With NORM the vector is RMS-normalised on the way in with the
-// reference's arithmetic (gpu_kernels.h:72-105):
-// o = half(x * (rsqrt(mean(x^2) + 1e-5) * w)).
 template <bool NORM>
-__device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const GemvParams& p, float* red) {
-    const int tid = threadIdx.x;
+struct XPieces {
+    u32x4 v[XP];
+    u32x4 w[NORM ? XP : 1];
+};
+
+template <int W, bool NORM>
+__device__ __forceinline__ void load_x(XPieces<NORM>& xr, const GemvParams& p) {
+    constexpr int T = W * 64;
     const int n8 = p.K >> 3;  // 8-half pieces of real data
     const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
+    const u32x4* wg = reinterpret_cast<const u32x4*>(p.norm_w);
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        const int e = min(i * T + (int)threadIdx.x, n8 - 1);  // clamped, masked in stage_x
+        xr.v[i] = xg[e];
+        if (NORM) xr.w[i] = wg[e];
+    }
+}
+
+// One piece of 8 halves: normalise (optional), permute, reduce the chunk constants over the 4 lanes of a chunk, store.
+template <bool NORM>
+__device__ __forceinline__ void stage_piece(u32x4* xs, float2* ab, const GemvParams& p, int e, u32x4 v, u32x4 wv, float ss,
+                                            bool store_norm) {
+    const int n8 = p.K >> 3;
+    if (e >= n8) v = u32x4{0u, 0u, 0u, 0u};
+    if (NORM) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const h16x2 h = as_h2(v[i]);
+            const h16x2 hw = as_h2(wv[i]);
+            h16x2 o;
+            o[0] = (h16_t)((float)h[0] * (ss * (float)hw[0]));
+            o[1] = (h16_t)((float)h[1] * (ss * (float)hw[1]));
+            v[i] = as_u32(o);
+        }
+        if (store_norm && e < n8) reinterpret_cast<u32x4*>(p.norm_out)[e] = v;
+    }
+    const h16x2 sixteenth = {(h16_t)0.0625f, (h16_t)0.0625f};
+    // v holds halves h0..h7 as (h0,h1)(h2,h3)(h4,h5)(h6,h7) -> (h0,h4)(h1,h5)(h2,h6)(h3,h7)
+    const h16x2 p0 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x05040100u));
+    const h16x2 p1 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x07060302u)) * sixteenth;
+    const h16x2 p2 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x05040100u));
+    const h16x2 p3 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x07060302u)) * sixteenth;
+    // fp32 sums of the stored halves: dot products against (1, 1)
+    const uint32_t ones = 0x3C003C00u;
+    const float even = dot2(as_u32(p0), ones, dot2(as_u32(p2), ones, 0.0f));
+    const float odd = dot2(as_u32(p1), ones, dot2(as_u32(p3), ones, 0.0f));
+    float a = fmaf(16.0f, odd, even);  // sum of the activations as the dot product sees them
+    float b = even + odd;              // sum of the stored fp16 values
+    // the 4 dword pieces of a chunk sit in 4 adjacent lanes
+    a += dpp_mov<0xB1>(a);
+    a += dpp_mov<0x4E>(a);
+    b += dpp_mov<0xB1>(b);
+    b += dpp_mov<0x4E>(b);
+    if (e < p.C * 4) {
+        u32x4 o = {as_u32(p0), as_u32(p1), as_u32(p2), as_u32(p3)};
+        xs[(e & 3) * p.C + (e >> 2)] = o;
+        if ((e & 3) == 0) ab[e >> 2] = make_float2(a, 1024.0f * b);
+    }
+}
+
+__device__ __forceinline__ float piece_sumsq(u32x4 v, float part) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const h16x2 h = as_h2(v[i]);
+        const float a = (float)h[0], b = (float)h[1];
+        part = fmaf(a, a, part);
+        part = fmaf(b, b, part);
+    }
+    return part;
+}
+
+template <int W, bool NORM>
+__device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const GemvParams& p, float* red, const XPieces<NORM>& xr) {
+    constexpr int T = W * 64;
+    const int tid = threadIdx.x;
+    const int n8 = p.K >> 3;
+    const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
+    const u32x4* wg = reinterpret_cast<const u32x4*>(p.norm_w);
     float ss = 0.0f;
     if (NORM) {
         float part = 0.0f;
-        for (int e = tid; e < n8; e += 256) {
-            const u32x4 v = xg[e];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const h16x2 h = as_h2(v[i]);
-                const float a = (float)h[0], b = (float)h[1];
-                part = fmaf(a, a, part);
-                part = fmaf(b, b, part);
-            }
-        }
+        for (int i = 0; i < XP; i++)
+            if (i * T + tid < n8) part = piece_sumsq(xr.v[i], part);
+        for (int e = XP * T + tid; e < n8; e += T) part = piece_sumsq(xg[e], part);
         part = wave_sum(part);
         if ((tid & 63) == 0) red[tid >> 6] = part;
         __syncthreads();
-        ss = (red[0] + red[1]) + (red[2] + red[3]);
+        float r[W];
+#pragma unroll
+        for (int i = 0; i < W; i++) r[i] = red[i];
+#pragma unroll
+        for (int n = W; n > 1; n >>= 1)
+#pragma unroll
+            for (int i = 0; i < n / 2; i++) r[i] = r[2 * i] + r[2 * i + 1];
+        ss = r[0];
         ss /= (float)p.K;
         ss += 1e-5f;
         ss = 1.0f / sqrtf(ss);
     }
-    const u32x4* wg = reinterpret_cast<const u32x4*>(p.norm_w);
-    u32x4* og = reinterpret_cast<u32x4*>(p.norm_out);
-    const bool store_norm = NORM && og != nullptr && blockIdx.x == 0 && blockIdx.y == 0;
-    const h16x2 sixteenth = {(h16_t)0.0625f, (h16_t)0.0625f};
-    for (int e0 = 0; e0 < p.C * 4; e0 += 256) {  // uniform trip count: the quad reduction below needs all lanes
-        const int e = e0 + tid;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (e < n8) {
-            v = xg[e];
-            if (NORM) {
-                const u32x4 wv = wg[e];
+    const bool store_norm = NORM && p.norm_out != nullptr && blockIdx.x == 0 && blockIdx.y == 0;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const h16x2 h = as_h2(v[i]);
-                    const h16x2 hw = as_h2(wv[i]);
-                    h16x2 o;
-                    o[0] = (h16_t)((float)h[0] * (ss * (float)hw[0]));
-                    o[1] = (h16_t)((float)h[1] * (ss * (float)hw[1]));
-                    v[i] = as_u32(o);
-                }
-                if (store_norm) og[e] = v;
-            }
-        }
-        // v holds halves h0..h7 as (h0,h1)(h2,h3)(h4,h5)(h6,h7) -> (h0,h4)(h1,h5)(h2,h6)(h3,h7)
-        const h16x2 p0 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x05040100u));
-        const h16x2 p1 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x07060302u)) * sixteenth;
-        const h16x2 p2 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x05040100u));
-        const h16x2 p3 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x07060302u)) * sixteenth;
-        const float even = ((float)p0[0] + (float)p0[1]) + ((float)p2[0] + (float)p2[1]);
-        const float odd = ((float)p1[0] + (float)p1[1]) + ((float)p3[0] + (float)p3[1]);
-        float a = fmaf(16.0f, odd, even);  // sum of the activations as the dot product sees them
-        float b = even + odd;              // sum of the stored fp16 values
-        // the 4 dword pieces of a chunk sit in 4 adjacent lanes
-        a += dpp_mov<0xB1>(a);
-        a += dpp_mov<0x4E>(a);
-        b += dpp_mov<0xB1>(b);
-        b += dpp_mov<0x4E>(b);
-        if (e < p.C * 4) {
-            u32x4 o = {as_u32(p0), as_u32(p1), as_u32(p2), as_u32(p3)};
-            xs[(e & 3) * p.C + (e >> 2)] = o;
-            if ((e & 3) == 0) ab[e >> 2] = make_float2(a, 1024.0f * b);
-        }
+    for (int i = 0; i < XP; i++)
+        if (i * T < p.C * 4)  // uniform: the quad reduction needs all lanes
+            stage_piece<NORM>(xs, ab, p, i * T + tid, xr.v[i], xr.w[NORM ? i : 0], ss, store_norm);
+    for (int e0 = XP * T; e0 < p.C * 4; e0 += T) {
+        const int e = e0 + tid;
+        const int ec = min(e, n8 - 1);
+        const u32x4 v = xg[ec];
+        u32x4 wv = v;
+        if (NORM) wv = wg[ec];
+        stage_piece<NORM>(xs, ab, p, e, v, wv, ss, store_norm);
     }
     __syncthreads();
 }
@@ -202,41 +226,52 @@ __device__ __forceinline__ int map_row(int li, int head_size) {
     return (pi / half) * head_size + (pi % half) + (li & 1) * half;
 }
 
-template <int R, int KIND, bool NORM, bool ROPE>
-__global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
+template <int W, int R, int D, int KIND, bool NORM, bool ROPE>
+__global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     extern __shared__ u32x4 xs[];
-    __shared__ float red[4];
+    __shared__ float red[W];
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: row addresses stay scalar
     const int C = p.C;
     const int pwh = C * 4;
     const int P = (C + 63) >> 6;  // 64-lane passes per row
     float2* ab = reinterpret_cast<float2*>(xs + 4 * C);
     const int which = (KIND == KIND_QKV) ? blockIdx.y : 0;
     const bool rope_here = ROPE && which != 2;
+    constexpr bool RES = KIND == KIND_SINGLE;
     uint32_t magic = 0x64006400u;  // fp16 pair (1024.0, 1024.0), kept in a VGPR
     asm("" : "+v"(magic));
 
     constexpr int NS = (KIND == KIND_FFN) ? 2 * R : R;
     const Int4Mat m0 = (KIND == KIND_QKV) ? (which == 0 ? p.m[0] : (which == 1 ? p.m[1] : p.m[2])) : p.m[0];
     const Int4Mat m1 = p.m[1];  // FFN: up
+    uint16_t* out = (KIND == KIND_QKV) ? (which == 0 ? p.out[0] : (which == 1 ? p.out[1] : p.out[2])) : p.out[0];
+    {
+        const int loff = (KIND == KIND_QKV) ? (which == 0 ? p.loff[0] : (which == 1 ? p.loff[1] : p.loff[2])) : p.loff[0];
+        if (loff != -1) out += (size_t)loff + (size_t)(*p.pos) * p.N;
+    }
 
-    // this workgroup's row groups
-    const int groups_total = (p.N + 4 * R - 1) / (4 * R);
+    // This workgroup's row groups (W waves x R rows each).  A wave walks its rows as a sequence of stages (group-major,
+    // then pass); D stages are in flight at any time.  The sequence is padded to a multiple of D with repeats of the
+    // last stage, which are loaded (same addresses again) but not accumulated, so that the number of loads between a
+    // stage's request and its use is a compile-time constant.
+    const int groups_total = (p.N + W * R - 1) / (W * R);
     const int g_begin = blockIdx.x * p.groups_per_wg;
     const int g_end = min(groups_total, g_begin + p.groups_per_wg);
-    const int total = (g_end - g_begin) * P;  // stages this wave walks through
+    const int total = (g_end - g_begin) * P;
 
     // ---- load cursor
     const uint32_t* wrow[NS];
     const uint32_t* zrow[NS];
     const uint16_t* srow[NS];
-    int lg = g_begin, lp = 0, lit = 0;
+    const uint16_t* resrow[R];
+    int lg = g_begin, lp = 0, ls = 0;
     auto set_rows = [&](int g) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const int li = min((g * 4 + wave) * R + r, p.N - 1);  // indices past N are recomputed, never stored
+            const int li = min((g * W + wave) * R + r, p.N - 1);  // indices past N are recomputed, never stored
             const int row = rope_here ? map_row<true>(li, p.head_size) : li;
+            resrow[r] = out + row;
             if (KIND == KIND_FFN) {
                 wrow[2 * r] = m0.w + (size_t)row * pwh;
                 zrow[2 * r] = m0.z + (size_t)row * p.pzh;
@@ -251,15 +286,30 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
             }
         }
     };
-    auto load_next = [&](Stage<NS>& st) {
-        if (lit < total) {
-            load_stage<NS>(st, wrow, zrow, srow, lp * 64 + lane, C);
-            lit++;
+    auto issue = [&](Stage<NS>& st) {
+        const int c = min(lp * 64 + lane, C - 1);  // lanes past the row end repeat its last chunk; consume() drops them
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            st.w[i] = load_nt(reinterpret_cast<const u32x4*>(wrow[i]) + c);
+#ifdef AWQ_PROBE_NOZS
+            st.zw[i] = 0x88888888u;
+            st.s[i] = 0x2000;
+#else
+            st.zw[i] = zrow[i][c >> 5];
+            st.s[i] = srow[i][c >> 2];
+#endif
+        }
+        if (RES) {
+#pragma unroll
+            for (int r = 0; r < R; r++) st.res[r] = *resrow[r];
+        }
+        ls++;
+        if (ls < total) {
             lp++;
             if (lp == P) {
                 lp = 0;
                 lg++;
-                if (lit < total) set_rows(lg);
+                set_rows(lg);
             }
         }
     };
@@ -269,27 +319,26 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
     for (int i = 0; i < NS; i++) sum[i] = 0.0f;
 
     // ---- consume cursor
-    int cg = g_begin, cp = 0;
-    auto finish_group = [&]() {
+    int cg = g_begin, cp = 0, cs = 0;
+    auto finish_group = [&](const Stage<NS>& st) {
+#ifndef AWQ_PROBE_NOREDUCE
 #pragma unroll
         for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]);
-        const int li0 = (cg * 4 + wave) * R;
+#endif
+        const int li0 = (cg * W + wave) * R;
         if (lane == 0 && li0 < p.N) {
-            uint16_t* out = (KIND == KIND_QKV) ? (which == 0 ? p.out[0] : (which == 1 ? p.out[1] : p.out[2])) : p.out[0];
-            const int loff = (KIND == KIND_QKV) ? (which == 0 ? p.loff[0] : (which == 1 ? p.loff[1] : p.loff[2])) : p.loff[0];
-            if (loff != -1) out += (size_t)loff + (size_t)(*p.pos) * p.N;
             if (rope_here) {
                 // q/k are rounded to fp16 and then rotated, as the separate RoPE kernel does (gpu_kernels.h:351-361)
                 const int half = p.head_size >> 1;
-                const float2* cs = p.rope + (size_t)(*p.pos) * half;
+                const float2* cs_tab = p.rope + (size_t)(*p.pos) * half;
 #pragma unroll
-                for (int r = 0; r < R; r += 2) {
+                for (int r = 0; r + 1 < R; r += 2) {
                     const int li = li0 + r;
                     if (li < p.N) {
                         const int row = map_row<true>(li, p.head_size);
                         const float v0 = half_bits_to_float(float_to_half_bits(sum[r]));
                         const float v1 = half_bits_to_float(float_to_half_bits(sum[r + 1]));
-                        const float2 c = cs[row % half];
+                        const float2 c = cs_tab[row % half];
                         out[row] = float_to_half_bits(v0 * c.x - v1 * c.y);
                         out[row + half] = float_to_half_bits(v0 * c.y + v1 * c.x);
                     }
@@ -307,7 +356,7 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
                             v = g * sum[2 * r + 1];
                         } else {
                             v = sum[r];
-                            if (KIND == KIND_SINGLE && p.accum) v += half_bits_to_float(out[row]) * p.inv_gpu_count;
+                            if (RES && p.accum) v += half_bits_to_float(st.res[r]) * p.inv_gpu_count;
                         }
                         out[row] = float_to_half_bits(v);
                     }
@@ -318,30 +367,58 @@ __global__ __launch_bounds__(256) void gemv_int4_kernel(const GemvParams p) {
         for (int i = 0; i < NS; i++) sum[i] = 0.0f;
     };
     auto consume = [&](const Stage<NS>& st) {
-        consume_stage<NS>(st, xs, ab, cp * 64 + lane, C, sum, magic);
-        cp++;
-        if (cp == P) {
-            finish_group();
-            cp = 0;
-            cg++;
+        if (cs < total) {
+            const int c = cp * 64 + lane;
+            const int cc = min(c, C - 1);
+            u32x4 xq[4];
+#ifdef AWQ_PROBE_NOLDS
+#pragma unroll
+            for (int qi = 0; qi < 4; qi++) xq[qi] = u32x4{magic, magic + qi, magic + cc, magic};
+            const float2 cab = make_float2(1.0f, 2.0f);
+#else
+#pragma unroll
+            for (int qi = 0; qi < 4; qi++) xq[qi] = xs[qi * C + cc];
+            const float2 cab = ab[cc];
+#endif
+            const int zshift = ((cc >> 2) & 7) * 4;
+#pragma unroll
+            for (int i = 0; i < NS; i++) {
+                const float zf = (float)((st.zw[i] >> zshift) & 0xFu);
+                const float acc = chunk_dot(st.w[i], zf, xq, cab.x, cab.y, magic);
+                const float sc = c < C ? half_bits_to_float(st.s[i]) : 0.0f;
+                sum[i] = fmaf(sc, acc, sum[i]);
+            }
+            cs++;
+            cp++;
+            if (cp == P) {
+                finish_group(st);
+                cp = 0;
+                cg++;
+            }
         }
     };
 
-    // The first two stages of packed weights are requested before x is staged, so that their HBM latency overlaps
-    // the staging (and the RMSNorm reduction); after that two stages stay in flight across row groups.
-    Stage<NS> a, b;
-    if (total > 0) set_rows(lg);
-    load_next(a);
-    load_next(b);
-    stage_x<NORM>(xs, ab, p, red);
-    for (int it = 0; it < total; it += 2) {
-        consume(a);
-        load_next(a);
-        if (it + 1 < total) {
-            consume(b);
-            load_next(b);
+    // The first D stages of packed weights are requested before x is staged, so that their HBM latency overlaps the
+    // staging (and the RMSNorm reduction).
+    XPieces<NORM> xr;
+    load_x<W, NORM>(xr, p);
+    Stage<NS> st[D];
+    set_rows(lg);
+#pragma unroll
+    for (int d = 0; d < D; d++) issue(st[d]);
+#ifndef AWQ_PROBE_NOSTAGE
+    stage_x<W, NORM>(xs, ab, p, red, xr);
+#endif
+    const int rounds = (total + D - 1) / D;
+    for (int r = 1; r < rounds; r++) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            consume(st[d]);
+            issue(st[d]);
         }
     }
+#pragma unroll
+    for (int d = 0; d < D; d++) consume(st[d]);
 }
 
 // out[n*K + k] = half_rne((q - z) * s): exact fp32 product, one rounding.
@@ -401,31 +478,80 @@ Int4Mat to_mat(const awq_qweight* w) { return Int4Mat{w->weight, w->zeros, w->sc
 
 bool qw_ok(const awq_qweight* w) { return w && w->weight && w->zeros && w->scales; }
 
-// Row groups per workgroup: enough workgroups to fill the chip several times over, but at least ~8 pipeline stages
-// per wave when the matrix is large enough to afford it (a stage = one 64-lane pass over the wave's rows).
-int pick_groups_per_wg(int groups_total, int passes) {
-    static int forced = -1;
-    if (forced < 0) {
-        const char* e = getenv("AWQ_GEMV_GROUPS_PER_WG");
-        forced = e ? atoi(e) : 0;
-    }
-    if (forced > 0) return forced;
-    int gpw = 1;
-    while (gpw * passes < 8 && groups_total / (gpw * 2) >= 512) gpw *= 2;
-    return gpw;
-}
+// Launch geometry of one matrix-vector product.
+struct GemvPlan {
+    int waves;   // waves per workgroup (4, 8)
+    int rows;    // rows per wave (1, 2, 4)
+    int depth;   // stages in flight per wave (2, 3, 4, 6)
+    int groups;  // row groups per workgroup
+};
 
-template <int R, int KIND, bool ROPE>
-int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
-    const int groups_total = div_up(p.N, 4 * R);
-    p.groups_per_wg = pick_groups_per_wg(groups_total, div_up(p.C, 64));
+template <int W, int R, int D, int KIND, bool ROPE>
+int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, int groups_per_wg) {
+    const int groups_total = div_up(p.N, W * R);
+    p.groups_per_wg = groups_per_wg;
     const dim3 grid(div_up(groups_total, p.groups_per_wg), grid_y);
     const size_t lds = (size_t)p.C * 72;  // activations + per-chunk constants
     if (p.norm_w)
-        hipLaunchKernelGGL((gemv_int4_kernel<R, KIND, true, ROPE>), grid, dim3(256), lds, ctx->stream, p);
+        hipLaunchKernelGGL((gemv_int4_kernel<W, R, D, KIND, true, ROPE>), grid, dim3(W * 64), lds, ctx->stream, p);
     else
-        hipLaunchKernelGGL((gemv_int4_kernel<R, KIND, false, ROPE>), grid, dim3(256), lds, ctx->stream, p);
+        hipLaunchKernelGGL((gemv_int4_kernel<W, R, D, KIND, false, ROPE>), grid, dim3(W * 64), lds, ctx->stream, p);
     return awq_check_launch(what);
+}
+
+template <int W, int R, int KIND, bool ROPE>
+int dispatch_depth(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, const GemvPlan& plan) {
+    constexpr int NS = (KIND == KIND_FFN) ? 2 * R : R;
+    int depth = plan.depth;
+    while (depth > 2 && (NS * depth > 16 || depth == 5 || depth == 7)) depth--;  // what the register file affords
+    switch (depth) {
+        case 2: return launch<W, R, 2, KIND, ROPE>(ctx, p, grid_y, what, plan.groups);
+        case 3: if constexpr (NS * 3 <= 16) return launch<W, R, 3, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
+        case 4: if constexpr (NS * 4 <= 16) return launch<W, R, 4, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
+        case 6: if constexpr (NS * 6 <= 16) return launch<W, R, 6, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
+        case 8: if constexpr (NS * 8 <= 16) return launch<W, R, 8, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
+    }
+    awq_set_error("no int4 matrix-vector kernel with %d stages in flight for %d streams", plan.depth, NS);
+    return AWQ_ERR_ARG;
+}
+
+// Tuning overrides for experiments: AWQ_GEMV_WAVES, AWQ_GEMV_ROWS, AWQ_GEMV_DEPTH, AWQ_GEMV_GROUPS_PER_WG.
+int env_int(const char* name) {
+    const char* e = getenv(name);
+    return e ? atoi(e) : 0;
+}
+
+// Measured on MI355X at the 7B shapes: one row (one gate/up pair) per wave, two passes in flight, 8 waves sharing the
+// staged activations; long rows (K > 8192) want 16 waves for the staging and a third pass in flight.
+GemvPlan plan_for(int K, int rows) {
+    GemvPlan plan;
+    plan.waves = K > 8192 ? 16 : 8;
+    plan.rows = rows;
+    plan.depth = K > 8192 ? 3 : 2;
+    plan.groups = 1;
+    return plan;
+}
+
+template <int KIND, bool ROPE>
+int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan plan) {
+    static const int forced_w = env_int("AWQ_GEMV_WAVES");
+    static const int forced_r = env_int("AWQ_GEMV_ROWS");
+    static const int forced_d = env_int("AWQ_GEMV_DEPTH");
+    static const int forced_g = env_int("AWQ_GEMV_GROUPS_PER_WG");
+    if (forced_w) plan.waves = forced_w;
+    if (forced_r) plan.rows = forced_r;
+    if (forced_d) plan.depth = forced_d;
+    if (forced_g) plan.groups = forced_g;
+    if (ROPE && plan.rows < 2) plan.rows = 2;  // a rotation pair lives in one wave
+#define AWQ_CASE(W_, R_) \
+    if (plan.waves == W_ && plan.rows == R_) return dispatch_depth<W_, R_, KIND, ROPE>(ctx, p, grid_y, what, plan);
+    AWQ_CASE(4, 2) AWQ_CASE(4, 4) AWQ_CASE(8, 2) AWQ_CASE(8, 4) AWQ_CASE(16, 2)
+    if constexpr (!ROPE) {
+        AWQ_CASE(4, 1) AWQ_CASE(8, 1) AWQ_CASE(16, 1)
+    }
+#undef AWQ_CASE
+    awq_set_error("no int4 matrix-vector kernel for %d waves x %d rows", plan.waves, plan.rows);
+    return AWQ_ERR_ARG;
 }
 
 }  // namespace
@@ -445,8 +571,7 @@ int awq_launch_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const
     p.norm_w = norm_w;
     p.norm_out = norm_out;
     // 2 rows per wave keep >= 2 workgroups per CU busy at N = 4096; 4 rows amortise staging on big N
-    if (N >= 8192) return launch<4, KIND_SINGLE, false>(ctx, p, 1, "gemv_int4");
-    return launch<2, KIND_SINGLE, false>(ctx, p, 1, "gemv_int4");
+    return dispatch<KIND_SINGLE, false>(ctx, p, 1, "gemv_int4", plan_for(K, 1));
 }
 
 int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
@@ -467,8 +592,8 @@ int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* val
     p.pos = pos;
     p.norm_w = norm_w;
     p.norm_out = norm_out;
-    if (rope) return launch<4, KIND_QKV, true>(ctx, p, 3, "qkv_matvec_rope");
-    return launch<4, KIND_QKV, false>(ctx, p, 3, "qkv_matvec");
+    if (rope) return dispatch<KIND_QKV, true>(ctx, p, 3, "qkv_matvec_rope", plan_for(K, 2));
+    return dispatch<KIND_QKV, false>(ctx, p, 3, "qkv_matvec", plan_for(K, 2));
 }
 
 int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w, const awq_qweight* up_w, int K,
@@ -480,7 +605,7 @@ int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qwe
     p.out[0] = out;
     p.norm_w = norm_w;
     p.norm_out = norm_out;
-    return launch<2, KIND_FFN, false>(ctx, p, 1, "ffn_matvec_silu");
+    return dispatch<KIND_FFN, false>(ctx, p, 1, "ffn_matvec_silu", plan_for(K, 1));
 }
 
 extern "C" {
