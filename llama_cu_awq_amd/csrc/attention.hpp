@@ -1,0 +1,127 @@
+// Single-workgroup attention for one head at short context (device function shared by the stand-alone kernel and
+// by the QKV matrix-vector kernel, whose last-arriving workgroup of a head runs it).
+//
+// What it computes is MultiHeadAttention of the reference for one head (gpu_kernels.h:368-451): scores
+// q.k * 1/sqrt(head_size) rounded to fp16, softmax over positions 0..pos in fp32 with the probabilities rounded to
+// fp16, then the probability-weighted sum of the value rows in fp32, stored as fp16.  The fp16 scores are also left
+// in att (the reference's att buffer holds them between its two phases).
+#pragma once
+
+#include "common.hpp"
+
+// Floats of LDS the function needs for a context of at most max_seq positions.
+__host__ __device__ constexpr int attention_head_lds_floats(int max_seq, int head_size, int waves) {
+    return ((max_seq + 3) & ~3) + waves * head_size + 2 * waves;
+}
+
+// LP = lanes per position (head_size / 8), NW = waves of the calling workgroup (all of them must call).
+// lds: attention_head_lds_floats() floats, free for use.  k_head / v_head: the head's slice of row 0 of the layer's
+// caches; rows are row_stride halves apart.
+template <int LP, int NW>
+__device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att_head, const uint16_t* q_head,
+                                               const uint16_t* k_head, const uint16_t* v_head, int head_size,
+                                               int row_stride, float alpha, int size, float* lds) {
+    constexpr int T = NW * 64;
+    float* sc = lds;                          // [size] scores (fp16-rounded values)
+    float* acc_lds = lds + ((size + 3) & ~3);  // [NW][head_size]
+    float* red = acc_lds + NW * head_size;     // [2 * NW]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int PW = 64 / LP;
+    const int j = lane % LP, pr = lane / LP;
+    const int tstep = NW * PW;  // positions covered by the workgroup per round
+    const int tfirst = wave * PW + pr;
+    const u32x4 qv = *reinterpret_cast<const u32x4*>(q_head + j * 8);
+    const uint16_t* kh = k_head + j * 8;
+    const uint16_t* vh = v_head + j * 8;
+    // The value rows of the first round are requested together with its key rows: at short context that is all of
+    // them, and the softmax then runs while they are on their way.
+    u32x4 vfirst[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int t = tfirst + k * tstep;
+        if (t < size) vfirst[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+    }
+    for (int t0 = tfirst; t0 - tfirst < size; t0 += 4 * tstep) {
+        u32x4 kv[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * tstep;
+            if (t < size) kv[k] = *reinterpret_cast<const u32x4*>(kh + (size_t)t * row_stride);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * tstep;
+            float s = 0.0f;
+            if (t < size) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) s = dot2(kv[k][i], qv[i], s);
+            }
+            s = group_sum<LP>(s);
+            if (j == 0 && t < size) {
+                const uint16_t hb = float_to_half_bits(s * alpha);
+                att_head[t] = hb;
+                sc[t] = half_bits_to_float(hb);
+            }
+        }
+    }
+    __syncthreads();
+    float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed (its softmax block has 1024 threads)
+    for (int t = tid; t < size; t += T) m = fmaxf(m, sc[t]);
+    m = wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = red[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) m = fmaxf(m, red[w]);
+    float sum = 0.0f;
+    for (int t = tid; t < size; t += T) sum += expf(sc[t] - m);
+    sum = wave_sum(sum);
+    if (lane == 0) red[NW + wave] = sum;
+    __syncthreads();
+    sum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) sum += red[NW + w];
+
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.0f;
+    for (int t0 = tfirst; t0 - tfirst < size; t0 += 4 * tstep) {
+        u32x4 vv[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * tstep;
+            if (t0 == tfirst)
+                vv[k] = vfirst[k];
+            else if (t < size)
+                vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = t0 + k * tstep;
+            if (t < size) {
+                const float e = expf(sc[t] - m);
+                const float pv = half_bits_to_float(float_to_half_bits(e / sum));
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const h16x2 hv = as_h2(vv[k][i]);
+                    acc[2 * i] = fmaf((float)hv[0], pv, acc[2 * i]);
+                    acc[2 * i + 1] = fmaf((float)hv[1], pv, acc[2 * i + 1]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        for (int off = LP; off < 64; off <<= 1) acc[i] += __shfl_xor(acc[i], off);
+    if (pr == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc_lds[wave * head_size + j * 8 + i] = acc[i];
+    }
+    __syncthreads();
+    if (tid < head_size) {
+        float total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; w++) total += acc_lds[w * head_size + tid];
+        out_head[tid] = float_to_half_bits(total);
+    }
+}

@@ -2,11 +2,11 @@
 // KV-cache attention, the fp16 classifier matrix-vector product and the greedy
 // sampler.  Arithmetic and rounding points follow the reference kernels cited
 // at each entry point; launch geometry and data movement are this library's.
+#include "attention.hpp"
 #include "common.hpp"
 
 namespace {
 
-constexpr int kAttnFusedMaxSeq = 512;  // up to this launch size attention runs as one workgroup per head
 
 // ------------------------------------------------------------------ embed
 __global__ __launch_bounds__(256) void embed_kernel(uint16_t* x, const uint16_t* table, int dim, const int* tokens,
@@ -229,100 +229,11 @@ __global__ __launch_bounds__(1024) void attn_fused_kernel(uint16_t* output, uint
                                                           const uint16_t* key_cache, const uint16_t* value_cache, int head_size,
                                                           int kv_mul, int row_stride, float alpha, const int* pPos) {
     extern __shared__ float fsm[];
-    float* sc = fsm;                // [size] scores (fp16-rounded values)
-    __shared__ float red[32];
     const int size = *pPos + 1;
-    float* acc_lds = fsm + ((size + 3) & ~3);  // [16][head_size]
     const int h = blockIdx.x;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    constexpr int PW = 64 / LP;
-    const int j = lane % LP, pr = lane / LP;
-    const int tstep = 16 * PW;  // positions covered by the workgroup per round
-    const int tfirst = wave * PW + pr;
-    const u32x4 qv = *reinterpret_cast<const u32x4*>(q + (size_t)h * head_size + j * 8);
-    const uint16_t* kh = key_cache + (size_t)(h / kv_mul) * head_size + j * 8;
-    const uint16_t* vh = value_cache + (size_t)(h / kv_mul) * head_size + j * 8;
-    uint16_t* a = att + (size_t)h * size;
-    for (int t0 = tfirst; t0 - tfirst < size; t0 += 4 * tstep) {
-        u32x4 kv[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int t = t0 + k * tstep;
-            if (t < size) kv[k] = *reinterpret_cast<const u32x4*>(kh + (size_t)t * row_stride);
-        }
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int t = t0 + k * tstep;
-            float s = 0.0f;
-            if (t < size) {
-#pragma unroll
-                for (int i = 0; i < 4; i++) s = dot2(kv[k][i], qv[i], s);
-            }
-            s = group_sum<LP>(s);
-            if (j == 0 && t < size) {
-                const uint16_t hb = float_to_half_bits(s * alpha);
-                a[t] = hb;
-                sc[t] = half_bits_to_float(hb);
-            }
-        }
-    }
-    __syncthreads();
-    float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed
-    for (int t = tid; t < size; t += 1024) m = fmaxf(m, sc[t]);
-    m = wave_max(m);
-    if (lane == 0) red[wave] = m;
-    __syncthreads();
-    m = red[0];
-#pragma unroll
-    for (int w = 1; w < 16; w++) m = fmaxf(m, red[w]);
-    float sum = 0.0f;
-    for (int t = tid; t < size; t += 1024) sum += expf(sc[t] - m);
-    sum = wave_sum(sum);
-    if (lane == 0) red[16 + wave] = sum;
-    __syncthreads();
-    sum = 0.0f;
-#pragma unroll
-    for (int w = 0; w < 16; w++) sum += red[16 + w];
-
-    float acc[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) acc[i] = 0.0f;
-    for (int t0 = tfirst; t0 - tfirst < size; t0 += 4 * tstep) {
-        u32x4 vv[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int t = t0 + k * tstep;
-            if (t < size) vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
-        }
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int t = t0 + k * tstep;
-            if (t < size) {
-                const float e = expf(sc[t] - m);
-                const float pv = half_bits_to_float(float_to_half_bits(e / sum));
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const h16x2 hv = as_h2(vv[k][i]);
-                    acc[2 * i] = fmaf((float)hv[0], pv, acc[2 * i]);
-                    acc[2 * i + 1] = fmaf((float)hv[1], pv, acc[2 * i + 1]);
-                }
-            }
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < 8; i++)
-        for (int off = LP; off < 64; off <<= 1) acc[i] += __shfl_xor(acc[i], off);
-    if (pr == 0) {
-#pragma unroll
-        for (int i = 0; i < 8; i++) acc_lds[wave * head_size + j * 8 + i] = acc[i];
-    }
-    __syncthreads();
-    if (tid < head_size) {
-        float total = 0.0f;
-#pragma unroll
-        for (int w = 0; w < 16; w++) total += acc_lds[w * head_size + tid];
-        output[(size_t)h * head_size + tid] = float_to_half_bits(total);
-    }
+    attention_head<LP, 16>(output + (size_t)h * head_size, att + (size_t)h * size, q + (size_t)h * head_size,
+                           key_cache + (size_t)(h / kv_mul) * head_size, value_cache + (size_t)(h / kv_mul) * head_size,
+                           head_size, row_stride, alpha, size, fsm);
 }
 
 // ------------------------------------------------------------------ fp16 matvec
@@ -440,13 +351,36 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* x, int siz
     const int tid = threadIdx.x;
     float best = -INFINITY;
     int best_i = 0x7FFFFFFF;
-    for (int i = tid; i < size; i += 1024) {
-        const float v = half_bits_to_float(x[i]);
-        if (v > best) {
+    auto take = [&](float v, int i) {
+        if (v > best || (v == best && i < best_i)) {
             best = v;
             best_i = i;
         }
+    };
+    // 8 logits per load, 4 loads in flight per thread (x is 16-byte aligned: it is a device allocation's start)
+    const int n8 = size >> 3;
+    const u32x4* x8 = reinterpret_cast<const u32x4*>(x);
+    for (int e0 = 0; e0 < n8; e0 += 4 * 1024) {
+        u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int e = e0 + k * 1024 + tid;
+            if (e < n8) v[k] = x8[e];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int e = e0 + k * 1024 + tid;
+            if (e < n8) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const h16x2 h = as_h2(v[k][i]);
+                    take((float)h[0], e * 8 + 2 * i);
+                    take((float)h[1], e * 8 + 2 * i + 1);
+                }
+            }
+        }
     }
+    for (int i = n8 * 8 + tid; i < size; i += 1024) take(half_bits_to_float(x[i]), i);
     for (int off = 32; off > 0; off >>= 1) {
         const float ov = __shfl_xor(best, off);
         const int oi = __shfl_xor(best_i, off);
@@ -486,7 +420,7 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
     const int row_stride = num_heads * head_size / kv_mul;
     const float alpha = (float)(1.0 / sqrt((double)head_size));
     if (max_seq_len <= kAttnFusedMaxSeq) {
-        const size_t lds = (size_t)(((max_seq_len + 3) & ~3) + 16 * head_size) * sizeof(float);
+        const size_t lds = (size_t)attention_head_lds_floats(max_seq_len, head_size, 16) * sizeof(float);
         hipLaunchKernelGGL((attn_fused_kernel<LP>), dim3(num_heads), dim3(1024), lds, ctx->stream, output, att, q, key_cache,
                            value_cache, head_size, kv_mul, row_stride, alpha, pos);
         return awq_check_launch("attn_fused");

@@ -17,6 +17,7 @@
 // OR-ing them into the mantissa of 1024.0, products are accumulated in fp32 by
 // v_dot2_f32_f16 with the 1024 offset and the zero point cancelled through
 // per-chunk constants, and the group scale is applied once per 32 elements.
+#include <math.h>
 #include <stdlib.h>
 
 #include "common.hpp"
@@ -114,7 +115,11 @@ __device__ __forceinline__ void load_x(XPieces<NORM>& xr, const GemvParams& p) {
     for (int i = 0; i < XP; i++) {
         const int e = min(i * T + (int)threadIdx.x, n8 - 1);  // clamped, masked in stage_x
         xr.v[i] = xg[e];
+#ifdef AWQ_PROBE_NOW
+        if (NORM) xr.w[i] = xr.v[i];
+#else
         if (NORM) xr.w[i] = wg[e];
+#endif
     }
 }
 
@@ -186,8 +191,10 @@ __device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const GemvParams&
             if (i * T + tid < n8) part = piece_sumsq(xr.v[i], part);
         for (int e = XP * T + tid; e < n8; e += T) part = piece_sumsq(xg[e], part);
         part = wave_sum(part);
+#ifndef AWQ_PROBE_NOBAR
         if ((tid & 63) == 0) red[tid >> 6] = part;
         __syncthreads();
+#endif
         float r[W];
 #pragma unroll
         for (int i = 0; i < W; i++) r[i] = red[i];
@@ -419,6 +426,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     }
 #pragma unroll
     for (int d = 0; d < D; d++) consume(st[d]);
+
 }
 
 // out[n*K + k] = half_rne((q - z) * s): exact fp32 product, one rounding.

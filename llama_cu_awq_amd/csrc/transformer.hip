@@ -472,7 +472,8 @@ int network_fused(awq_transformer* t, int seq_len_bin) {
     const int kv_mul = p.n_heads / p.n_kv_heads;
     int* pPos = s.pos;
     int r;
-    if ((r = awq_embed(ctx, s.x, t->embed, dim, s.shared_tokens, pPos))) return r;
+    // the token list's device mirror (kept by reset / set_pos / accept / the sampler) saves a read over PCIe
+    if ((r = awq_embed(ctx, s.x, t->embed, dim, t->tokens_dev, pPos))) return r;
     for (int l = 0; l < p.n_layers; l++) {
         const awq_layer_weights& L = t->layers[l];
         const int loff = l * p.seq_len * kv_dim;
