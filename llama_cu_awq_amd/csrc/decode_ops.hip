@@ -115,11 +115,11 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(uint16_t* att, const u
     }
 }
 
-// Pass 2: softmax statistics (recomputed by every workgroup of a head from the
-// fp16 scores: a few KB), probabilities rounded to fp16 as the reference
-// does, and P.V over this workgroup's slice of positions.  With more than one
-// split the per-split partial sums are combined, in split order, by the last
-// workgroup of the head to arrive.
+// Pass 2: softmax statistics (recomputed by every workgroup of a head from the fp16 scores: a few KB),
+// probabilities rounded to fp16 as the reference does, and P.V over this workgroup's slice of positions.  The slice
+// is sized so that its value rows are requested in one go, before the statistics are computed.  With more than one
+// split the per-split partial sums are written through to memory and combined, in split order, by the last workgroup
+// of the head to arrive.
 template <int LP>
 __global__ __launch_bounds__(256) void attn_softmax_pv_kernel(uint16_t* output, const uint16_t* att,
                                                               const uint16_t* value_cache, int head_size, int kv_mul,
@@ -137,22 +137,16 @@ __global__ __launch_bounds__(256) void attn_softmax_pv_kernel(uint16_t* output, 
     const int wave = tid >> 6;
     const uint16_t* a = att + (size_t)h * size;
 
-    // max (the reference seeds idle threads of its 1024-thread block with 0)
-    float m = (size < 1024) ? 0.0f : -INFINITY;
-    for (int t = tid; t < size; t += 256) m = fmaxf(m, half_bits_to_float(a[t]));
-    m = wave_max(m);
-    if (lane == 0) red[wave] = m;
-    __syncthreads();
-    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    __syncthreads();
-    float sum = 0.0f;
-    for (int t = tid; t < size; t += 256) sum += expf(half_bits_to_float(a[t]) - m);
-    sum = wave_sum(sum);
-    if (lane == 0) red[wave] = sum;
-    __syncthreads();
-    sum = (red[0] + red[1]) + (red[2] + red[3]);
-
-    // this workgroup's positions
+    // the head's scores: 8 per thread requested together cover 2048 positions, a loop takes the rest.  They are
+    // requested ahead of the value rows because loads return in order and the statistics need only the scores.
+    constexpr int SP = 8;
+    uint16_t sv[SP];
+#pragma unroll
+    for (int i = 0; i < SP; i++) {
+        const int t = i * 256 + tid;
+        sv[i] = a[min(t, size - 1)];
+    }
+    // this workgroup's positions; a round covers 64 of them (4 waves x PW positions x 4 loads per lane)
     const int per = (size + nsplit - 1) / nsplit;
     const int tb = split * per;
     const int te = min(size, tb + per);
@@ -160,22 +154,61 @@ __global__ __launch_bounds__(256) void attn_softmax_pv_kernel(uint16_t* output, 
     const int j = lane % LP;
     const int pr = lane / LP;
     const uint16_t* vh = value_cache + (size_t)(h / kv_mul) * head_size + j * 8;
+    const int tfirst = tb + wave * PW + pr;
+    u32x4 vfirst[4];
+    uint16_t afirst[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int t = tfirst + k * 4 * PW;
+        if (t < te) {
+            vfirst[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+            afirst[k] = a[t];
+        }
+    }
+
+    // max (the reference seeds idle threads of its 1024-thread block with 0)
+    float m = (size < 1024) ? 0.0f : -INFINITY;
+#pragma unroll
+    for (int i = 0; i < SP; i++)
+        if (i * 256 + tid < size) m = fmaxf(m, half_bits_to_float(sv[i]));
+    for (int t = SP * 256 + tid; t < size; t += 256) m = fmaxf(m, half_bits_to_float(a[t]));
+    m = wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < SP; i++)
+        if (i * 256 + tid < size) sum += expf(half_bits_to_float(sv[i]) - m);
+    for (int t = SP * 256 + tid; t < size; t += 256) sum += expf(half_bits_to_float(a[t]) - m);
+    sum = wave_sum(sum);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    sum = (red[0] + red[1]) + (red[2] + red[3]);
+
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.0f;
-    // four rows per lane are requested before any is used (each is an HBM/L2 round trip)
-    for (int t0 = tb + wave * PW + pr; t0 - pr - wave * PW < te; t0 += 16 * PW) {
+    for (int t0 = tfirst; t0 - pr - wave * PW < te; t0 += 16 * PW) {
         u32x4 vv[4];
+        uint16_t av[4];
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const int t = t0 + k * 4 * PW;
-            if (t < te) vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+            if (t0 == tfirst) {
+                vv[k] = vfirst[k];
+                av[k] = afirst[k];
+            } else if (t < te) {
+                vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+                av[k] = a[t];
+            }
         }
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const int t = t0 + k * 4 * PW;
             if (t < te) {
-                const float e = expf(half_bits_to_float(a[t]) - m);
+                const float e = expf(half_bits_to_float(av[k]) - m);
                 const float p = half_bits_to_float(float_to_half_bits(e / sum));  // probability rounded to fp16
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -203,18 +236,26 @@ __global__ __launch_bounds__(256) void attn_softmax_pv_kernel(uint16_t* output, 
         if (tid < head_size) output[(size_t)h * head_size + tid] = float_to_half_bits(total);
         return;
     }
+    // Publish this split's partial sums: written through at agent scope (a release fence per workgroup would flush
+    // the whole L2 each time), waited for, then counted in.
     float* my = partial + ((size_t)h * kAttnMaxSplits + split) * kAttnMaxHeadSize;
-    if (tid < head_size) my[tid] = total;
-    __threadfence();
+    if (tid < head_size) __hip_atomic_store(&my[tid], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (tid == 0) arrival = atomicAdd(&counter[h], 1u);
+    if (tid == 0) arrival = __hip_atomic_fetch_add(&counter[h], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (arrival == (unsigned int)(nsplit - 1)) {
-        __threadfence();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         if (tid < head_size) {
             const float* ph = partial + (size_t)h * kAttnMaxSplits * kAttnMaxHeadSize;
+            // all partials are requested before the first is used (each is a trip to memory)
+            float pv[kAttnMaxSplits];
+#pragma unroll
+            for (int sp = 0; sp < kAttnMaxSplits; sp++) pv[sp] = sp < nsplit ? ph[(size_t)sp * kAttnMaxHeadSize + tid] : 0.0f;
             float s = 0.0f;
-            for (int sp = 0; sp < nsplit; sp++) s += ph[(size_t)sp * kAttnMaxHeadSize + tid];
+#pragma unroll
+            for (int sp = 0; sp < kAttnMaxSplits; sp++)
+                if (sp < nsplit) s += pv[sp];
             output[(size_t)h * head_size + tid] = float_to_half_bits(s);
         }
         if (tid == 0) counter[h] = 0;  // ready for the next launch
@@ -428,7 +469,7 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
     hipLaunchKernelGGL((attn_scores_kernel<LP>), dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, ctx->stream, att, q,
                        key_cache, head_size, kv_mul, row_stride, alpha, pos);
     if (int r = awq_check_launch("attn_scores")) return r;
-    int nsplit = div_up(max_seq_len, 256);
+    int nsplit = div_up(max_seq_len, 64);  // one round of value rows per workgroup
     if (nsplit > kAttnMaxSplits) nsplit = kAttnMaxSplits;
     if (nsplit < 1) nsplit = 1;
     hipLaunchKernelGGL((attn_softmax_pv_kernel<LP>), dim3(nsplit, num_heads), dim3(256), 0, ctx->stream, output, att,

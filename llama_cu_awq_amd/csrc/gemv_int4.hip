@@ -6,17 +6,15 @@
 // followed by one of the epilogues (plain store, KV-cache row store, fused
 // residual add, SiLU(gate)*up).
 //
-// How: a workgroup of 4 waves stages the activation vector once in LDS
-// (optionally applying RMSNorm on the way in), pre-permuted so that a lane's
-// 32 consecutive K elements (one 16-byte load of packed weights, the same lane
-// ownership as the reference's uint4 load) meet their activations as packed
-// fp16 pairs.  Each wave owns R consecutive rows and walks the row in passes
-// of 64 x 16 bytes; two passes of loads are kept in flight, the first two
-// requested before staging starts; a lane reads its activations from LDS once
-// per pass and reuses them for the R rows.  Nibbles become fp16 numbers by
-// OR-ing them into the mantissa of 1024.0, products are accumulated in fp32 by
-// v_dot2_f32_f16 with the 1024 offset and the zero point cancelled through
-// per-chunk constants, and the group scale is applied once per 32 elements.
+// How: a workgroup of W waves (8, or 16 for long rows) stages the activation vector once in LDS (optionally applying
+// RMSNorm on the way in), pre-permuted so that a lane's 32 consecutive K elements (one 16-byte load of packed
+// weights, the same lane ownership as the reference's uint4 load) meet their activations as packed fp16 pairs.
+// Each wave owns R consecutive rows (one gate/up pair in the fused FFN form) and walks them in passes of 64 x 16
+// bytes with D passes in flight.  Loads return in order, so a wave first requests its share of the activations,
+// then its first D passes of weights, and stages the activations while the weights are still on their way.
+// Nibbles become fp16 numbers by OR-ing them into the mantissa of 1024.0, products are accumulated in fp32 by
+// v_dot2_f32_f16 with the 1024 offset and the zero point cancelled through per-chunk constants, and the group scale
+// is applied once per 32 elements.
 #include <math.h>
 #include <stdlib.h>
 
@@ -65,10 +63,7 @@ __device__ __forceinline__ float chunk_dot(const u32x4 w, const float zf, const 
                                            const uint32_t magic) {
     float acc = fmaf(-zf, A, -B);
 #pragma unroll
-#ifndef AWQ_PROBE_QI
-#define AWQ_PROBE_QI 4
-#endif
-    for (int qi = 0; qi < AWQ_PROBE_QI; qi++) {
+    for (int qi = 0; qi < 4; qi++) {
         const uint32_t d = w[qi];
         const uint32_t d8 = d >> 8;
         acc = dot2((d & 0x000F000Fu) | magic, xq[qi][0], acc);
@@ -115,11 +110,7 @@ __device__ __forceinline__ void load_x(XPieces<NORM>& xr, const GemvParams& p) {
     for (int i = 0; i < XP; i++) {
         const int e = min(i * T + (int)threadIdx.x, n8 - 1);  // clamped, masked in stage_x
         xr.v[i] = xg[e];
-#ifdef AWQ_PROBE_NOW
-        if (NORM) xr.w[i] = xr.v[i];
-#else
         if (NORM) xr.w[i] = wg[e];
-#endif
     }
 }
 
@@ -191,10 +182,8 @@ __device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const GemvParams&
             if (i * T + tid < n8) part = piece_sumsq(xr.v[i], part);
         for (int e = XP * T + tid; e < n8; e += T) part = piece_sumsq(xg[e], part);
         part = wave_sum(part);
-#ifndef AWQ_PROBE_NOBAR
         if ((tid & 63) == 0) red[tid >> 6] = part;
         __syncthreads();
-#endif
         float r[W];
 #pragma unroll
         for (int i = 0; i < W; i++) r[i] = red[i];
@@ -298,13 +287,8 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
 #pragma unroll
         for (int i = 0; i < NS; i++) {
             st.w[i] = load_nt(reinterpret_cast<const u32x4*>(wrow[i]) + c);
-#ifdef AWQ_PROBE_NOZS
-            st.zw[i] = 0x88888888u;
-            st.s[i] = 0x2000;
-#else
             st.zw[i] = zrow[i][c >> 5];
             st.s[i] = srow[i][c >> 2];
-#endif
         }
         if (RES) {
 #pragma unroll
@@ -328,10 +312,8 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     // ---- consume cursor
     int cg = g_begin, cp = 0, cs = 0;
     auto finish_group = [&](const Stage<NS>& st) {
-#ifndef AWQ_PROBE_NOREDUCE
 #pragma unroll
         for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]);
-#endif
         const int li0 = (cg * W + wave) * R;
         if (lane == 0 && li0 < p.N) {
             if (rope_here) {
@@ -378,15 +360,9 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
             const int c = cp * 64 + lane;
             const int cc = min(c, C - 1);
             u32x4 xq[4];
-#ifdef AWQ_PROBE_NOLDS
-#pragma unroll
-            for (int qi = 0; qi < 4; qi++) xq[qi] = u32x4{magic, magic + qi, magic + cc, magic};
-            const float2 cab = make_float2(1.0f, 2.0f);
-#else
 #pragma unroll
             for (int qi = 0; qi < 4; qi++) xq[qi] = xs[qi * C + cc];
             const float2 cab = ab[cc];
-#endif
             const int zshift = ((cc >> 2) & 7) * 4;
 #pragma unroll
             for (int i = 0; i < NS; i++) {
@@ -413,9 +389,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     set_rows(lg);
 #pragma unroll
     for (int d = 0; d < D; d++) issue(st[d]);
-#ifndef AWQ_PROBE_NOSTAGE
     stage_x<W, NORM>(xs, ab, p, red, xr);
-#endif
     const int rounds = (total + D - 1) / D;
     for (int r = 1; r < rounds; r++) {
 #pragma unroll
@@ -490,7 +464,7 @@ bool qw_ok(const awq_qweight* w) { return w && w->weight && w->zeros && w->scale
 struct GemvPlan {
     int waves;   // waves per workgroup (4, 8)
     int rows;    // rows per wave (1, 2, 4)
-    int depth;   // stages in flight per wave (2, 3, 4, 6)
+    int depth;   // stages in flight per wave (2, 3, 4)
     int groups;  // row groups per workgroup
 };
 
@@ -511,13 +485,11 @@ template <int W, int R, int KIND, bool ROPE>
 int dispatch_depth(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, const GemvPlan& plan) {
     constexpr int NS = (KIND == KIND_FFN) ? 2 * R : R;
     int depth = plan.depth;
-    while (depth > 2 && (NS * depth > 16 || depth == 5 || depth == 7)) depth--;  // what the register file affords
+    while (depth > 2 && (NS * depth > 16 || depth > 4)) depth--;  // what the register file affords
     switch (depth) {
         case 2: return launch<W, R, 2, KIND, ROPE>(ctx, p, grid_y, what, plan.groups);
         case 3: if constexpr (NS * 3 <= 16) return launch<W, R, 3, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
         case 4: if constexpr (NS * 4 <= 16) return launch<W, R, 4, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
-        case 6: if constexpr (NS * 6 <= 16) return launch<W, R, 6, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
-        case 8: if constexpr (NS * 8 <= 16) return launch<W, R, 8, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
     }
     awq_set_error("no int4 matrix-vector kernel with %d stages in flight for %d streams", plan.depth, NS);
     return AWQ_ERR_ARG;
