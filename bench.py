@@ -231,13 +231,13 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_int4_kernel<2, FFN> (fused gate/up + SiLU*mul), K=%d N=%d" % (dim, hid),
+            "kernel": "gemv_int4_kernel<8 waves, 1 row pair, 2 passes in flight, FFN> (fused gate/up + SiLU*mul), K=%d N=%d" % (dim, hid),
             "achieved": round(ffn_gbps, 1),
             "peak": HBM_PEAK / 1e9,
             "unit": "GB/s",
             "frac": round(ffn_gbps * 1e9 / HBM_PEAK, 4),
             # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE (7B shape; profiles/gemv_int4_ffn_7b_pmc.md)
-            "traffic": 47048704 if (dim, hid) == (4096, 11008) else None,
+            "traffic": 47063305 if (dim, hid) == (4096, 11008) else None,
             "bytes_per_launch": ffn_bytes,
             "us_per_launch": round(ffn_us, 3),
         },
