@@ -19,10 +19,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 namespace pf {
 
-constexpr int BM = 128;      // tokens per tile
-constexpr int BN = 128;      // weight rows per tile
-constexpr int BK = 32;       // K per step = one 16-byte packed chunk per weight row
-constexpr int LDS_ROW = 40;  // halves per LDS tile row (32 + 8 padding)
+constexpr int BM = 128;  // tokens per tile
+constexpr int BN = 128;  // weight rows per tile
+constexpr int BK = 64;   // K per step: 128 bytes of fp16 per LDS tile row
 
 enum Epi { EPI_STORE = 0, EPI_RESID = 1, EPI_QKV = 2, EPI_FFN = 3 };
 
@@ -35,6 +34,7 @@ struct GemmParams {
     int N[3];  // rows of each matrix
     int C, pzh, sh;
     int epi;
+    int mtiles, ntiles;
     uint16_t* out[3];
     long long ldo[3];       // output row stride in elements
     long long out_off[3];   // element offset of output row 0 (KV cache: loff + pos0 * kv_dim)
@@ -63,57 +63,120 @@ __device__ __forceinline__ u32x4 dequant8(uint32_t d, uint32_t z, h16x2 s2) {
     return u32x4{as_u32(t0 * s2), as_u32(t1 * s2), as_u32(t2 * s2), as_u32(t3 * s2)};  // one rounding each
 }
 
-// Which matrix / row a tile row maps to, and where its output goes.
-struct TileMap {
-    int mat[2];   // matrix of tile rows [0,64) and [64,128)
-    int row0[2];  // first matrix row of each half
+// A tile's 128 columns are four blocks of 32 weight rows.  Which matrix a block belongs to and its first row:
+// single / QKV: consecutive rows of one matrix; FFN: blocks alternate gate, up over the same 32 row indices, so that a
+// wave (two adjacent blocks) holds a gate column and its up column in the same lane.
+struct BlockMap {
+    int mat, row0;
 };
 
-__device__ __forceinline__ TileMap tile_map(const GemmParams& p, int tile) {
-    TileMap t;
-    if (p.epi == EPI_FFN) {  // 64 gate rows + the 64 up rows of the same indices
-        t.mat[0] = 0;
-        t.mat[1] = 1;
-        t.row0[0] = t.row0[1] = tile * 64;
-    } else {
-        int m = 0, tt = tile;
-        if (p.epi == EPI_QKV) {
-            const int t0 = p.N[0] / BN, t1 = p.N[1] / BN;
-            if (tt >= t0 + t1) {
-                m = 2;
-                tt -= t0 + t1;
-            } else if (tt >= t0) {
-                m = 1;
-                tt -= t0;
-            }
-        }
-        t.mat[0] = t.mat[1] = m;
-        t.row0[0] = tt * BN;
-        t.row0[1] = tt * BN + 64;
+__device__ __forceinline__ BlockMap block_map(const GemmParams& p, int tile, int b) {
+    BlockMap m;
+    if (p.epi == EPI_FFN) {
+        m.mat = b & 1;
+        m.row0 = tile * 64 + (b >> 1) * 32;
+        return m;
     }
-    return t;
+    int mat = 0, tt = tile;
+    if (p.epi == EPI_QKV) {
+        const int t0 = p.N[0] / BN, t1 = p.N[1] / BN;
+        if (tt >= t0 + t1) {
+            mat = 2;
+            tt -= t0 + t1;
+        } else if (tt >= t0) {
+            mat = 1;
+            tt -= t0;
+        }
+    }
+    m.mat = mat;
+    m.row0 = tt * BN + b * 32;
+    return m;
 }
 
-__global__ __launch_bounds__(256) void gemm_int4_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDS_ROW];
-    __shared__ __attribute__((aligned(16))) uint16_t Ws[2][BN * LDS_ROW];
+// The activation tile in LDS is [128 rows][64 halves] with the 16-byte chunk index XOR-ed with a key of the row, so
+// that a wave's fragment reads (32 consecutive rows, one chunk) spread over all banks without padding.
+__device__ __forceinline__ int lds_key(int row) { return (row ^ (row >> 3)) & 7; }
+__device__ __forceinline__ int lds_off(int row, int chunk) { return row * BK + ((chunk ^ lds_key(row)) << 3); }
+
+constexpr int A_STAGES = 3;                   // activation tiles in the LDS ring (2 steps ahead)
+constexpr int W_STAGES = 3;                   // pairs of steps (one quantisation group) of packed weights in the LDS ring
+constexpr int TILE_BYTES = BM * BK * 2;       // 16 KB
+constexpr int W_WAVE_BYTES = 32 * 64 + 256 + 256;  // per wave and pair of steps: 32 rows x 64 packed bytes, zeros, scales
+constexpr int W_STAGE_BYTES = 4 * W_WAVE_BYTES;
+constexpr int GEMM_LDS_BYTES = A_STAGES * TILE_BYTES + W_STAGES * W_STAGE_BYTES;
+
+// Direct global -> LDS loads: lane L's 16 (4) bytes land at lds_byte_off + 16 (4) * L.  Issued as inline assembly,
+// so the compiler's wait-count bookkeeping does not see them; the kernel counts and waits for them itself.
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_byte_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_byte_off), "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void dma4(const void* gptr, uint32_t lds_byte_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_byte_off), "v"(gptr) : "memory");
+}
+
+// inverse of permute8: (h0,h4)(h1,h5)(h2,h6)(h3,h7) -> (h0,h1)(h2,h3)(h4,h5)(h6,h7)
+__device__ __forceinline__ u32x4 unpermute8(const u32x4 v) {
+    u32x4 o;
+    o[0] = __builtin_amdgcn_perm(v[1], v[0], 0x05040100u);
+    o[1] = __builtin_amdgcn_perm(v[3], v[2], 0x05040100u);
+    o[2] = __builtin_amdgcn_perm(v[1], v[0], 0x07060302u);
+    o[3] = __builtin_amdgcn_perm(v[3], v[2], 0x07060302u);
+    return o;
+}
+
+// C[m][n] = sum_k A[m][k] * half((q[n][k] - z) * s), tile 128 x 128, K step 64.
+//  * Workgroup = 4 waves; wave w owns tile columns 32w .. 32w+31 and all 128 rows: four 32x32x16 fp16 MFMA
+//    accumulators.  A lane's MFMA operand for the weights is 8 consecutive K of one weight row = one packed dword, so
+//    dequantised weights never pass through LDS: lane (row l % 32, half l / 32) takes its row's 16 packed bytes of
+//    the step and dequantises a dword right before the MFMAs that use it (bit-exact half((q-z)*s)).
+//  * Every global load is a direct global -> LDS load.  The activation tile (16 KB, natural order, read by every
+//    wave as fragments) travels two steps ahead into a ring of three tiles.  Packed weights travel per pair of steps
+//    (128 K = one quantisation group: 64 contiguous bytes per row, one zero-point dword and one scale) two pairs
+//    ahead into a ring that only the loading wave reads back, so they need no barrier.  LDS is the prefetch ring: no
+//    register carries a load across iterations and one hand-counted s_waitcnt per step covers everything.
+//  * One barrier per step.  The loop body has no conditional around its loads (steps past the end re-read the last
+//    ones with zero scales), so the number of loads between a request and its use is constant.
+// Workgroup ids are mapped so that the M tiles sharing a weight tile run on one XCD (ids go round-robin over the 8
+// XCDs), which reads the weights from HBM once.
+__global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];  // [A ring][W ring]; nothing else is in LDS
+    constexpr uint32_t W_RING = A_STAGES * TILE_BYTES;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int m0 = blockIdx.x * BM;
-    const TileMap tm = tile_map(p, blockIdx.y);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int tile = (slot / p.mtiles) * 8 + xcd;
+    if (tile >= p.ntiles) return;
+    const int m0 = (slot % p.mtiles) * BM;
 
-    // loader role: 2 threads per tile row, 16 K elements each
-    const int lrow = tid >> 1, lhalf = tid & 1;
-    const int am = m0 + lrow;
-    const bool a_ok = am < p.M;
-    const uint16_t* a_ptr = p.A + (size_t)(a_ok ? am : 0) * p.lda + lhalf * 16;
-    const int whalf = lrow >> 6;
-    const int wmat = tm.mat[whalf];
-    const int wrow = tm.row0[whalf] + (lrow & 63);
-    const uint32_t* wbase = (wmat == 0 ? p.w[0] : (wmat == 1 ? p.w[1] : p.w[2])) + (size_t)wrow * (p.C * 4) + lhalf * 2;
-    const uint32_t* zbase = (wmat == 0 ? p.z[0] : (wmat == 1 ? p.z[1] : p.z[2])) + (size_t)wrow * p.pzh;
-    const uint16_t* sbase = (wmat == 0 ? p.s[0] : (wmat == 1 ? p.s[1] : p.s[2])) + (size_t)wrow * p.sh;
+    // activation loader: wave w, instruction q covers tile rows (4w + q) * 8 .. + 8 (8 lanes x 16 bytes per row);
+    // the lane's LDS chunk is lane & 7, so it fetches the source chunk that the swizzle maps there
+    const uint16_t* a_src[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int r = (wave * 4 + q) * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ lds_key(r);
+        a_src[q] = p.A + (size_t)min(m0 + r, p.M - 1) * p.lda + c * 8;  // rows past M are computed, never stored
+    }
+    // weight loader: instruction q of a pair of steps covers the wave's rows 16q .. 16q+15, 4 lanes x 16 bytes per
+    // row; 16-byte unit u of a row's 64 bytes sits at LDS unit u ^ ((row >> 1) & 3) (bank spread for the reads below)
+    const BlockMap wb = block_map(p, tile, wave);
+    const uint32_t* wmat = (wb.mat == 0 ? p.w[0] : (wb.mat == 1 ? p.w[1] : p.w[2]));
+    const uint32_t* zmat = (wb.mat == 0 ? p.z[0] : (wb.mat == 1 ? p.z[1] : p.z[2]));
+    const uint16_t* smat = (wb.mat == 0 ? p.s[0] : (wb.mat == 1 ? p.s[1] : p.s[2]));
+    const uint32_t* w_src[2];
+    int w_unit[2];
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+        const int r = 16 * q + (lane >> 2);
+        w_unit[q] = (lane & 3) ^ ((r >> 1) & 3);
+        w_src[q] = wmat + (size_t)(wb.row0 + r) * (p.C * 4);
+    }
+    // consumer side: this lane's weight row and which 32-element half of a step it multiplies
+    const int lrow = lane & 31, lhalf = lane >> 5;
+    const uint32_t* zrow = zmat + (size_t)(wb.row0 + lrow) * p.pzh;
+    const size_t s_row = (size_t)(wb.row0 + lrow) * p.sh;  // index of the row's first scale (scales travel as aligned dwords)
+    const int n_groups = p.sh;
 
     f32x16 acc[4];
 #pragma unroll
@@ -121,83 +184,126 @@ __global__ __launch_bounds__(256) void gemm_int4_kernel(const GemmParams p) {
 #pragma unroll
         for (int j = 0; j < 16; j++) acc[i][j] = 0.0f;
 
-    const int nsteps = p.K / BK;
-    u32x4 ra0, ra1;
-    u32x2 rw;
-    uint32_t rz;
-    uint16_t rs;
-    auto gload = [&](int step) {
-        const int k0 = step * BK;
-        if (a_ok) {
-            ra0 = *reinterpret_cast<const u32x4*>(a_ptr + k0);
-            ra1 = *reinterpret_cast<const u32x4*>(a_ptr + k0 + 8);
-        } else {
-            ra0 = ra1 = u32x4{0u, 0u, 0u, 0u};
-        }
-        rw = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(wbase + (size_t)step * 4));
-        const int g = step >> 2;
-        rz = (zbase[g >> 3] >> (4 * (g & 7))) & 0xFu;
-        rs = sbase[g];
+    const int nsteps = (p.K + BK - 1) / BK;
+    const int k_last = (nsteps - 1) * BK;
+    auto load_a = [&](int step) {  // 4 loads
+        const int k0 = min(step * BK, k_last);
+        const uint32_t dst = (uint32_t)((step % A_STAGES) * TILE_BYTES + wave * 4096);
+#pragma unroll
+        for (int q = 0; q < 4; q++) dma16(a_src[q] + k0, dst + q * 1024);
     };
-    auto lstore = [&](int buf) {
-        u32x4* ad = reinterpret_cast<u32x4*>(&As[buf][lrow * LDS_ROW + lhalf * 16]);
-        ad[0] = permute8(ra0);
-        ad[1] = permute8(ra1);
-        const h16_t sh = __builtin_bit_cast(h16_t, rs);
+    auto load_w = [&](int pair) {  // 4 loads: K range [128 * pair, 128 * pair + 128) of the wave's 32 rows
+        const uint32_t dst = W_RING + (uint32_t)((pair % W_STAGES) * W_STAGE_BYTES + wave * W_WAVE_BYTES);
+#pragma unroll
+        for (int q = 0; q < 2; q++) dma16(w_src[q] + (size_t)min(pair * 4 + w_unit[q], p.C - 1) * 4, dst + q * 1024);
+        const int g = min(pair, n_groups - 1);
+        dma4(zrow + (g >> 3), dst + 2048);
+        dma4(smat + ((s_row + g) & ~(size_t)1), dst + 2304);
+    };
+    // K mapping of the four MFMAs of a step: MFMA j multiplies K chunk j (lanes 0-31) and chunk 4 + j (lanes 32-63),
+    // i.e. dword j of each lane's 16 bytes against the matching 8 activations.
+    auto compute = [&](int step) {
+        const uint16_t* at = reinterpret_cast<const uint16_t*>(lds_bytes + (step % A_STAGES) * TILE_BYTES);
+        const int pair = step >> 1;
+        const uint8_t* ws = lds_bytes + W_RING + (pair % W_STAGES) * W_STAGE_BYTES + wave * W_WAVE_BYTES;
+        const int unit = (step & 1) * 2 + lhalf;
+        const u32x4 wq = *reinterpret_cast<const u32x4*>(ws + lrow * 64 + ((unit ^ ((lrow >> 1) & 3)) << 4));
+        const uint32_t zw = *reinterpret_cast<const uint32_t*>(ws + 2048 + lane * 4);
+        const uint32_t sw = *reinterpret_cast<const uint32_t*>(ws + 2304 + lane * 4);
+        const int g = min(pair, n_groups - 1);
+        const uint32_t z = (zw >> (4 * (g & 7))) & 0xFu;
+        const uint16_t sbits = (uint16_t)(((s_row + g) & 1) ? (sw >> 16) : (sw & 0xFFFFu));
+        const bool live = step * BK + lhalf * 32 < p.K;  // past K: zero scale, zero products
+        const h16_t sh = __builtin_bit_cast(h16_t, live ? sbits : (uint16_t)0);
         const h16x2 s2 = {sh, sh};
-        u32x4* wd = reinterpret_cast<u32x4*>(&Ws[buf][lrow * LDS_ROW + lhalf * 16]);
-        wd[0] = dequant8(rw[0], rz, s2);
-        wd[1] = dequant8(rw[1], rz, s2);
-    };
-
-    gload(0);
-    lstore(0);
-    __syncthreads();
-    for (int step = 0; step < nsteps; step++) {
-        const int buf = step & 1;
-        if (step + 1 < nsteps) gload(step + 1);
-        // wave w: token rows 32w..32w+31 against all 128 weight rows
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-            const int koff = ks * 16 + (lane >> 5) * 8;
-            const h16x8 af = *reinterpret_cast<const h16x8*>(&As[buf][(wave * 32 + (lane & 31)) * LDS_ROW + koff]);
+        for (int j = 0; j < 4; j++) {
+            const h16x8 bf = __builtin_bit_cast(h16x8, unpermute8(dequant8(wq[j], z, s2)));
+            const int chunk = j + 4 * lhalf;
 #pragma unroll
-            for (int nb = 0; nb < 4; nb++) {
-                const h16x8 bf = *reinterpret_cast<const h16x8*>(&Ws[buf][(nb * 32 + (lane & 31)) * LDS_ROW + koff]);
-                acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, acc[nb], 0, 0, 0);
+            for (int i = 0; i < 4; i++) {
+                const h16x8 af = *reinterpret_cast<const h16x8*>(&at[lds_off(i * 32 + (lane & 31), chunk)]);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, acc[i], 0, 0, 0);
             }
         }
-        if (step + 1 < nsteps) lstore(buf ^ 1);
+    };
+
+    // Prologue: activation tiles 0, 1 and weight pairs 0, 1.
+    load_a(0);
+    load_a(1);
+    load_w(0);
+    load_w(1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int step = 0; step < nsteps; step += 2) {
+        // even step: request activation tile step+2 and weight pair (step/2)+2, then multiply
+        load_a(step + 2);  // into the slot that step-1 multiplied: every wave is past the barrier that ended it
+        load_w((step >> 1) + 2);  // into the slot this wave finished reading at the end of the previous iteration
+        compute(step);
+        // needed next: activation tile step+1, requested in the previous iteration's odd half, followed by 4 + 4
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        __syncthreads();
+        // odd step
+        load_a(step + 3);
+        compute(step + 1);
+        // needed next: activation tile step+2 (followed by 4 + 4 loads) and weight pair (step/2)+1 (older still)
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         __syncthreads();
     }
 
-    // epilogue: acc[nb][j] is D[row = 8*(j/4) + 4*(lane/32) + j%4][col = lane%32] of the 32x32 block
+    // epilogue: acc[i][j] is D[row = 32*i + 8*(j/4) + 4*(lane/32) + j%4][col = lane%32] of the wave's 32 columns
     const int col = lane & 31;
+    if (p.epi == EPI_FFN) {
+        // waves 0, 2 hold gate columns, waves 1, 3 the up columns of the same row indices: the up waves pass their
+        // accumulators through LDS once the loads still in flight have landed there
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        float* xch = reinterpret_cast<float*>(lds_bytes);  // [2 pairs][64 values][64 lanes]
+        if (wave & 1) {
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
-        const int m = m0 + wave * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
-        if (m >= p.M) continue;
-        if (p.epi == EPI_FFN) {
+            for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++) {
-                float g = acc[nb][j];
-                g *= 1.0f / (1.0f + expf(-g));
-                const float v = g * acc[nb + 2][j];
-                p.out[0][(size_t)p.out_off[0] + (size_t)m * p.ldo[0] + tm.row0[0] + nb * 32 + col] = float_to_half_bits(v);
+                for (int j = 0; j < 16; j++) xch[((wave >> 1) * 64 + i * 16 + j) * 64 + lane] = acc[i][j];
+        }
+        __syncthreads();
+        if (!(wave & 1)) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    const int m = m0 + i * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+                    if (m >= p.M) continue;
+                    float g = acc[i][j];
+                    g *= 1.0f / (1.0f + expf(-g));
+                    const float v = g * xch[((wave >> 1) * 64 + i * 16 + j) * 64 + lane];
+                    p.out[0][(size_t)p.out_off[0] + (size_t)m * p.ldo[0] + wb.row0 + col] = float_to_half_bits(v);
+                }
             }
-        } else {
+        }
+        return;
+    }
+    const int mat = wb.mat;
+    uint16_t* o = (mat == 0 ? p.out[0] : (mat == 1 ? p.out[1] : p.out[2])) +
+                  (size_t)(mat == 0 ? p.out_off[0] : (mat == 1 ? p.out_off[1] : p.out_off[2])) + wb.row0 + col;
+    const size_t ld = (size_t)(mat == 0 ? p.ldo[0] : (mat == 1 ? p.ldo[1] : p.ldo[2]));
 #pragma unroll
-            for (int nb = 0; nb < 4; nb++) {
-                const int hsel = nb >> 1;
-                const int mat = tm.mat[hsel];
-                const int n = tm.row0[hsel] + (nb & 1) * 32 + col;
-                uint16_t* o = (mat == 0 ? p.out[0] : (mat == 1 ? p.out[1] : p.out[2]));
-                const size_t idx = (size_t)(mat == 0 ? p.out_off[0] : (mat == 1 ? p.out_off[1] : p.out_off[2])) +
-                                   (size_t)m * (mat == 0 ? p.ldo[0] : (mat == 1 ? p.ldo[1] : p.ldo[2])) + n;
-                float v = acc[nb][j];
-                if (p.epi == EPI_RESID) v += half_bits_to_float(o[idx]);
-                o[idx] = float_to_half_bits(v);
+    for (int i = 0; i < 4; i++) {
+        // residual form: all 16 old values are requested before the first is used
+        uint16_t old[16];
+        if (p.epi == EPI_RESID) {
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                const int m = m0 + i * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+                old[j] = o[(size_t)min(m, p.M - 1) * ld];
             }
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int m = m0 + i * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+            if (m >= p.M) continue;
+            float v = acc[i][j];
+            if (p.epi == EPI_RESID) v += half_bits_to_float(old[j]);
+            o[(size_t)m * ld] = float_to_half_bits(v);
         }
     }
 }
@@ -365,8 +471,22 @@ __global__ __launch_bounds__(256) void copy_row_kernel(uint16_t* dst, const uint
 }  // namespace pf
 
 // ---------------------------------------------------------------- launchers (internal)
-static int launch_gemm(awq_ctx* ctx, const pf::GemmParams& p, int ntiles, const char* what) {
-    hipLaunchKernelGGL(pf::gemm_int4_kernel, dim3(div_up(p.M, pf::BM), ntiles), dim3(256), 0, ctx->stream, p);
+static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* what) {
+    static bool lds_raised = false;  // the kernel's 80 KB of LDS exceed the default dynamic limit
+    if (!lds_raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)pf::gemm_int4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           pf::GEMM_LDS_BYTES);
+        if (e != hipSuccess) {
+            awq_set_error("hipFuncSetAttribute(gemm_int4) failed: %s", hipGetErrorString(e));
+            return AWQ_ERR_HIP;
+        }
+        lds_raised = true;
+    }
+    p.mtiles = div_up(p.M, pf::BM);
+    p.ntiles = ntiles;
+    // ids go round-robin over the 8 XCDs; each XCD takes every 8th weight tile with all of its M tiles
+    const int grid = 8 * p.mtiles * div_up(ntiles, 8);
+    hipLaunchKernelGGL(pf::gemm_int4_kernel, dim3(grid), dim3(256), pf::GEMM_LDS_BYTES, ctx->stream, p);
     return awq_check_launch(what);
 }
 
