@@ -458,6 +458,125 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(uint16_t* out, const 
     }
 }
 
+// Causal attention on the matrix cores for 128-wide heads: 32 consecutive query tokens of one head per workgroup.
+// Same rounding points as above.
+//  1. S = Q K^T: both MFMA operands are 8 consecutive head dims of a row, so q and k rows are loaded straight from
+//     memory into fragments; wave w takes key blocks w, w+4, ...; scores go to LDS as fp16.
+//  2. softmax per query row over its causal range, probabilities written back to LDS as fp16 (zero past the range).
+//  3. O = P V: the weights operand needs 8 consecutive keys of one head dim, so value rows are transposed 8 x 8 in
+//     registers on their way into LDS (64 keys per tile, next tile's rows in flight during the multiply); wave w
+//     produces head dims 32w .. 32w+31.
+constexpr int AQ = 32;        // queries per workgroup
+constexpr int VT_STRIDE = 72; // halves per row of the transposed value tile (64 keys + 8 padding)
+
+__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, const uint16_t* q, const uint16_t* key_cache,
+                                                                const uint16_t* value_cache, int num_heads, int kv_mul, int M,
+                                                                int pos0, int s_stride) {
+    constexpr int HS = 128;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    uint16_t* S = reinterpret_cast<uint16_t*>(smem);                          // [AQ][s_stride]
+    uint16_t* Vt = reinterpret_cast<uint16_t*>(smem + AQ * s_stride * 2);     // [2][HS][VT_STRIDE]
+    const int h = blockIdx.y;
+    const int mq0 = blockIdx.x * AQ;
+    const int nq = min(AQ, M - mq0);
+    const int nk = pos0 + mq0 + nq;          // keys visible to the last query of the block
+    const int nk_pad = (nk + 63) & ~63;      // <= s_stride - 8
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kv_dim = num_heads * HS / kv_mul;
+    const float alpha = (float)(1.0 / sqrt((double)HS));
+    const uint16_t* kh = key_cache + (size_t)(h / kv_mul) * HS;
+    const uint16_t* vh = value_cache + (size_t)(h / kv_mul) * HS;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    // 1. scores
+    h16x8 qf[8];
+    {
+        const uint16_t* qrow = q + ((size_t)min(mq0 + l32, M - 1) * num_heads + h) * HS + lh * 8;
+#pragma unroll
+        for (int f = 0; f < 8; f++) qf[f] = *reinterpret_cast<const h16x8*>(qrow + f * 16);
+    }
+    for (int kb = wave; kb * 32 < nk_pad; kb += 4) {
+        const uint16_t* krow = kh + (size_t)min(kb * 32 + l32, nk - 1) * kv_dim + lh * 8;
+        h16x8 kf[8];
+#pragma unroll
+        for (int f = 0; f < 8; f++) kf[f] = *reinterpret_cast<const h16x8*>(krow + f * 16);
+        f32x16 acc;
+#pragma unroll
+        for (int j = 0; j < 16; j++) acc[j] = 0.0f;
+#pragma unroll
+        for (int f = 0; f < 8; f++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[f], kf[f], acc, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int row = (j >> 2) * 8 + lh * 4 + (j & 3);
+            S[row * s_stride + kb * 32 + l32] = float_to_half_bits(acc[j] * alpha);
+        }
+    }
+    __syncthreads();
+    // 2. softmax per query row (wave w takes rows w, w+4, ...); rows past nq get all-zero probabilities
+    for (int qi = wave; qi < AQ; qi += 4) {
+        const int size = qi < nq ? pos0 + mq0 + qi + 1 : 0;
+        float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed
+        for (int t = lane; t < size; t += 64) m = fmaxf(m, half_bits_to_float(S[qi * s_stride + t]));
+        m = wave_max(m);
+        float sum = 0.0f;
+        for (int t = lane; t < size; t += 64) sum += expf(half_bits_to_float(S[qi * s_stride + t]) - m);
+        sum = wave_sum(sum);
+        for (int t = lane; t < nk_pad; t += 64) {
+            float pv = 0.0f;
+            if (t < size) pv = expf(half_bits_to_float(S[qi * s_stride + t]) - m) / sum;
+            S[qi * s_stride + t] = float_to_half_bits(pv);
+        }
+    }
+    // 3. O = P V.  Loader role (threads 0..127): 8 keys x 8 dims, transposed in registers.
+    const int kg = tid & 7, dc = (tid >> 3) & 15;
+    const bool loader = tid < 128;
+    u32x4 vr[8];
+    auto load_v = [&](int t0) {
+        if (loader) {
+#pragma unroll
+            for (int r = 0; r < 8; r++)
+                vr[r] = *reinterpret_cast<const u32x4*>(vh + (size_t)min(t0 + kg * 8 + r, nk - 1) * kv_dim + dc * 8);
+        }
+    };
+    auto store_v = [&](int buf) {
+        if (loader) {
+            uint16_t* vt = Vt + buf * (HS * VT_STRIDE);
+#pragma unroll
+            for (int d = 0; d < 8; d++) {
+                const uint32_t sel = (d & 1) ? 0x07060302u : 0x05040100u;
+                u32x4 o;
+#pragma unroll
+                for (int r2 = 0; r2 < 4; r2++) o[r2] = __builtin_amdgcn_perm(vr[2 * r2 + 1][d >> 1], vr[2 * r2][d >> 1], sel);
+                *reinterpret_cast<u32x4*>(&vt[(dc * 8 + d) * VT_STRIDE + kg * 8]) = o;
+            }
+        }
+    };
+    f32x16 oacc;
+#pragma unroll
+    for (int j = 0; j < 16; j++) oacc[j] = 0.0f;
+    load_v(0);
+    store_v(0);
+    __syncthreads();  // also orders the probabilities written above
+    for (int t0 = 0, buf = 0; t0 < nk_pad; t0 += 64, buf ^= 1) {
+        const bool more = t0 + 64 < nk_pad;
+        if (more) load_v(t0 + 64);
+        const uint16_t* vt = Vt + buf * (HS * VT_STRIDE);
+#pragma unroll
+        for (int kc = 0; kc < 4; kc++) {
+            const h16x8 pf = *reinterpret_cast<const h16x8*>(&S[l32 * s_stride + t0 + kc * 16 + lh * 8]);
+            const h16x8 vf = *reinterpret_cast<const h16x8*>(&vt[(wave * 32 + l32) * VT_STRIDE + kc * 16 + lh * 8]);
+            oacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(pf, vf, oacc, 0, 0, 0);
+        }
+        if (more) store_v(buf ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const int row = (j >> 2) * 8 + lh * 4 + (j & 3);
+        if (row < nq) out[((size_t)(mq0 + row) * num_heads + h) * HS + wave * 32 + l32] = float_to_half_bits(oacc[j]);
+    }
+}
+
 __global__ void set_pos_kernel(int* pos_dev, volatile int* pos_host, int value) {
     *pos_dev = value;
     *pos_host = value;
@@ -557,6 +676,25 @@ int awq_launch_rope_rows(awq_ctx* ctx, uint16_t* q, uint16_t* kcache_layer, int 
 
 int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, const uint16_t* kc, const uint16_t* vc, int nh, int hs,
                             int kv_mul, int M, int pos0) {
+    if (hs == 128) {
+        const int s_stride = ((pos0 + M + 63) & ~63) + 8;
+        const size_t lds = (size_t)pf::AQ * s_stride * 2 + 2 * 128 * pf::VT_STRIDE * 2;
+        if (lds > 160 * 1024) {
+            awq_set_error("prefill attention: context of %d positions does not fit in LDS", pos0 + M);
+            return AWQ_ERR_SHAPE;
+        }
+        if (lds > 64 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void*)pf::attn_prefill_mfma_kernel,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) {
+                awq_set_error("hipFuncSetAttribute(attn_prefill_mfma) failed: %s", hipGetErrorString(e));
+                return AWQ_ERR_HIP;
+            }
+        }
+        hipLaunchKernelGGL(pf::attn_prefill_mfma_kernel, dim3(div_up(M, pf::AQ), nh), dim3(256), lds, ctx->stream, out, q, kc, vc,
+                           nh, kv_mul, M, pos0, s_stride);
+        return awq_check_launch("attn_prefill_mfma");
+    }
     const int nk_max = (pos0 + M + 7) & ~7;
     const size_t lds = (size_t)pf::BQ * hs * 2 + (size_t)pf::BQ * nk_max * 2 + pf::BQ * 8;
     if (lds > 160 * 1024) {

@@ -43,9 +43,11 @@ def test_gemm_shape_guard(ctx):
 
 CFG = dict(dim=512, hidden_dim=1536, n_layers=3, n_heads=4, n_kv_heads=4, vocab_size=1024, seq_len=192, rope_theta=10000.0)
 CFG_GQA = dict(dim=512, hidden_dim=1280, n_layers=2, n_heads=8, n_kv_heads=2, vocab_size=512, seq_len=96, rope_theta=10000.0)
+# 128-wide heads with grouped KV: the matrix-core attention kernel with kv_mul > 1
+CFG_GQA128 = dict(dim=1024, hidden_dim=1536, n_layers=2, n_heads=8, n_kv_heads=2, vocab_size=512, seq_len=128, rope_theta=10000.0)
 
 
-@pytest.mark.parametrize("cfg,n_prompt", [(CFG, 130), (CFG, 16), (CFG, 1), (CFG_GQA, 70)])
+@pytest.mark.parametrize("cfg,n_prompt", [(CFG, 130), (CFG, 16), (CFG, 1), (CFG, 97), (CFG_GQA, 70), (CFG_GQA128, 75)])
 def test_prefill_matches_token_by_token_oracle(ctx, cfg, n_prompt):
     img = synth.make_model_image(cfg, seed=31)
     t = A.Transformer(ctx, image=img)
