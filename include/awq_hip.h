@@ -202,6 +202,34 @@ int awq_transformer_forward_logits(awq_transformer* t, int use_graph, int mode);
  * p = pos + 1; if write_token, tokens[p] = token; pos = p (pinned-host and device copies). */
 int awq_transformer_accept(awq_transformer* t, int token, int write_token);
 
+/* ---- temperature / top-p sampling on the GPU (the non-greedy branch of sample(), sampler.h:85-115) ---- */
+
+/* softmax_logits_kernel (gpu_kernels.h:507-557), in place: logits = half(logits / temperature), then
+ * p = half(float(half(expf(l - max))) / sum) with the sum taken over the unrounded exponentials in fp32. */
+int awq_softmax_logits(awq_ctx* ctx, uint16_t* logits, int size, float temperature);
+/* The reference's sort + prefix sum + sample_top_p_kernel (sampler.h:94-115, gpu_kernels.h:562-592) in one launch:
+ * sorted != 0 orders the fp16 probabilities descending (stable, as the reference's radix sort), sorted == 0 keeps
+ * index order; the token is the first position whose inclusive prefix sum, rounded to fp16, is >= threshold
+ * (position size-1 when none is).  The prefix sums are exact (fp16 values are multiples of 2^-24) and rounded once;
+ * the reference's CUB scan adds in fp16 in an unspecified order.  Then p = pos + 1; tokens[p] = token; pos = p
+ * (pinned-host and device copies).  probs is left untouched.  size <= 65535. */
+int awq_sample_top_p(awq_ctx* ctx, const uint16_t* probs, int size, float threshold, int sorted, int* tokens,
+                     volatile int* pos_host, int* pos_dev);
+
+/* Sampler (sampler.h:10-47): hyperparameters and the xorshift* state (sampler.h:65-74). */
+typedef struct awq_sampler awq_sampler;
+int awq_sampler_create(awq_ctx* ctx, int vocab_size, float temperature, float topp, unsigned long long rng_seed,
+                       awq_sampler** out);
+int awq_sampler_destroy(awq_sampler* sampler);
+/* sample() (sampler.h:77-115): draws the coin (every call, as the reference does), then the greedy kernel when
+ * temperature == 0 or gen_token == 0, else softmax + top-p (threshold coin * topp) or plain sampling (threshold coin
+ * when topp <= 0 or >= 1).  logits are overwritten on the non-greedy branch. */
+int awq_sampler_sample(awq_sampler* sampler, uint16_t* logits, int* tokens, volatile int* pos_host, int* pos_dev,
+                       int gen_token);
+/* The same on a transformer's own logits and token list (also keeps the device mirror of the token list current):
+ * run_transformer() = awq_transformer_forward_logits + awq_transformer_sample (llama2_q4.cu:541-601). */
+int awq_transformer_sample(awq_transformer* t, awq_sampler* sampler, int gen_token);
+
 /* ---- multi-token prefill.  No counterpart in the reference, which consumes the prompt one token per forward pass
  * (llama2_q4.cu:716-735); the contract is the state that loop would leave. ---- */
 

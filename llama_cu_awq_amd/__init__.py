@@ -4,6 +4,7 @@ from .ops import (  # noqa: F401
     Context,
     DeviceBuffer,
     QWeight,
+    Sampler,
     MultiHeadAttention,
     RoPERotation,
     argmax_advance,
@@ -15,5 +16,7 @@ from .ops import (  # noqa: F401
     matmul_q,
     qkv_matvec,
     rmsnorm,
+    sample_top_p,
+    softmax_logits,
 )
 from .model import Transformer, SCHEDULE_FUSED, SCHEDULE_PERSISTENT, SCHEDULE_REFERENCE  # noqa: F401

@@ -84,6 +84,12 @@ PROTOTYPES = {
     "awq_transformer_forward_logits": [_vp, _i, _i],
     "awq_transformer_accept": [_vp, _i, _i],
     "awq_transformer_trace": [_vp, _i, C.POINTER(C.c_longlong), _i, C.POINTER(C.c_int)],
+    "awq_softmax_logits": [_vp, _vp, _i, _f],
+    "awq_sample_top_p": [_vp, _vp, _i, _f, _i, _vp, _vp, _vp],
+    "awq_sampler_create": [_vp, _i, _f, _f, C.c_ulonglong, _pvp],
+    "awq_sampler_destroy": [_vp],
+    "awq_sampler_sample": [_vp, _vp, _vp, _vp, _vp, _i],
+    "awq_transformer_sample": [_vp, _vp, _i],
 }
 NON_STATUS = {"awq_last_error": ([], C.c_char_p), "awq_ctx_stream": ([_vp], _vp)}
 

@@ -52,62 +52,6 @@ static long time_in_ms() {
     return t.tv_sec * 1000 + t.tv_nsec / 1000000;
 }
 
-// xorshift* of the reference's sampler (sampler.h:65-74)
-static unsigned int random_u32(unsigned long long* state) {
-    *state ^= *state >> 12;
-    *state ^= *state << 25;
-    *state ^= *state >> 27;
-    return (unsigned int)((*state * 0x2545F4914F6CDD1Dull) >> 32);
-}
-static float random_f32(unsigned long long* state) { return (random_u32(state) >> 8) / 16777216.0f; }
-
-// ---- fp16 helpers for the host-side sampler
-static float h2f(uint16_t h) {
-    _Float16 v;
-    memcpy(&v, &h, 2);
-    return (float)v;
-}
-static uint16_t f2h(float f) {
-    _Float16 v = (_Float16)f;
-    uint16_t h;
-    memcpy(&h, &v, 2);
-    return h;
-}
-
-// Temperature / top-p sampling with the reference's arithmetic (sampler.h:85-115, gpu_kernels.h:507-592): logits
-// scaled and softmaxed with fp16 roundings in between, sorted descending (stable), prefix-summed in fp16, first index
-// whose prefix reaches coin*topp (coin when topp is off).  Runs on the host over a copy of the logits.
-static int sample_top_p(std::vector<uint16_t>& logits, float temperature, float topp, float coin) {
-    const int n = (int)logits.size();
-    for (int i = 0; i < n; i++) logits[i] = f2h(h2f(logits[i]) / temperature);
-    float max_val = -3.402823466e38f;
-    for (int i = 0; i < n; i++) max_val = std::max(max_val, h2f(logits[i]));
-    float sum = 0.0f;
-    for (int i = 0; i < n; i++) {
-        const float v = expf(h2f(logits[i]) - max_val);
-        logits[i] = f2h(v);
-        sum += v;
-    }
-    for (int i = 0; i < n; i++) logits[i] = f2h(h2f(logits[i]) / sum);
-    std::vector<int> idx(n);
-    for (int i = 0; i < n; i++) idx[i] = i;
-    float threshold = coin;
-    if (topp > 0 && topp < 1) {
-        std::stable_sort(idx.begin(), idx.end(), [&](int a, int b) { return h2f(logits[a]) > h2f(logits[b]); });
-        threshold = coin * topp;
-    }
-    uint16_t run = f2h(0.0f);
-    int pick = n - 1;
-    for (int i = 0; i < n; i++) {
-        run = f2h(h2f(run) + h2f(logits[idx[i]]));
-        if (h2f(run) >= threshold) {
-            pick = i;
-            break;
-        }
-    }
-    return idx[pick];
-}
-
 int main(int argc, char* argv[]) {
     // get_and_print_gpu_info(), llama2_q4.cu:817-837
     int device_count = 0;
@@ -233,8 +177,9 @@ int main(int argc, char* argv[]) {
     awq_run_state st;
     die_awq(awq_transformer_state(t, &st));
     die_awq(awq_transformer_reset(t, prompt_tokens.data(), num_prompt_tokens));
-    unsigned long long rng_state = rng_seed;
-    std::vector<uint16_t> host_logits(cfg.vocab_size);
+    // build_sampler(), llama2_q4.cu:922: the sampler owns the xorshift* state and runs on the GPU
+    awq_sampler* sampler = nullptr;
+    die_awq(awq_sampler_create(ctx, cfg.vocab_size, temperature, topp, rng_seed, &sampler));
     int token = prompt_tokens[0];
     int next;
     int pos = 0;
@@ -242,7 +187,6 @@ int main(int argc, char* argv[]) {
     if (batched_prompt && num_prompt_tokens > 1 && temperature == 0.0f) {
         // one batched pass over the prompt; echo it as the token-by-token loop would have
         const int n = std::min(num_prompt_tokens, steps);
-        for (int i = 0; i < n; i++) (void)random_f32(&rng_state);
         die_awq(awq_transformer_prefill(t, n, n == num_prompt_tokens));
         for (pos = 1; pos < n; pos++) {
             next = prompt_tokens[pos];
@@ -254,14 +198,13 @@ int main(int argc, char* argv[]) {
     while (pos < steps) {
         die_awq(awq_stream_sync(ctx));  // wait for the previous token, then launch the next before printing
         const bool gen_token = pos >= num_prompt_tokens - 1;
-        const float coin = random_f32(&rng_state);  // drawn every step, greedy or not (sampler.h:79)
-        if (temperature == 0.0f || !gen_token) {
+        if (temperature == 0.0f) {
+            // network + greedy sampler as one (graph-replayed) unit; the coin the reference draws anyway is never used
             die_awq(awq_transformer_forward(t, gen_token, use_graph, mode));
         } else {
+            // run_transformer(), llama2_q4.cu:541-601: the network, then sample() (greedy while the prompt is consumed)
             die_awq(awq_transformer_forward_logits(t, use_graph, mode == AWQ_SCHEDULE_PERSISTENT ? AWQ_SCHEDULE_FUSED : mode));
-            die_awq(awq_memcpy_d2h(ctx, host_logits.data(), st.logits, (size_t)cfg.vocab_size * 2));
-            const int sampled = sample_top_p(host_logits, temperature, topp, coin);
-            die_awq(awq_transformer_accept(t, sampled, 1));
+            die_awq(awq_transformer_sample(t, sampler, gen_token));
         }
         if (pos > 0) {
             next = st.shared_tokens[pos];
@@ -280,6 +223,7 @@ int main(int argc, char* argv[]) {
     printf("\n");
     printf("\n[GPU: %d] achieved tok/s: %f. Tokens: %d, seconds: %g\n", 0, timed_tokens / secs, timed_tokens, secs);
 
+    die_awq(awq_sampler_destroy(sampler));
     die_awq(awq_transformer_free(t));
     die_awq(awq_ctx_destroy(ctx));
     return 0;

@@ -25,6 +25,9 @@ int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const 
                           const uint16_t* norm_w, uint16_t* norm_out);
 int awq_launch_argmax(awq_ctx* ctx, const uint16_t* logits, int size, int* tokens, volatile int* pos_host, int* pos_dev,
                       int write_token, int* tokens_mirror);
+// sampler.hip
+int awq_sampler_run(awq_sampler* s, uint16_t* logits, int* tokens, volatile int* pos_host, int* pos_dev, int gen_token,
+                    int* mirror);
 // prefill.hip
 int awq_launch_gemm_single(awq_ctx* ctx, uint16_t* out, long long ldo, const uint16_t* A, int lda, int M, const awq_qweight* w,
                            int K, int N, int accum);
@@ -800,6 +803,14 @@ int awq_transformer_accept(awq_transformer* t, int token, int write_token) {
     hipLaunchKernelGGL(accept_kernel, dim3(1), dim3(1), 0, ctx->stream, token, t->s.shared_tokens, t->tokens_dev, t->s.shared_pos,
                        t->s.pos, write_token);
     return awq_check_launch("accept");
+}
+
+int awq_transformer_sample(awq_transformer* t, awq_sampler* sampler, int gen_token) {
+    AWQ_REQUIRE(t && sampler, AWQ_ERR_ARG, "null transformer or sampler");
+    awq_ctx* ctx = t->ctx;
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(t->shared->pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+    return awq_sampler_run(sampler, t->s.logits, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token, t->tokens_dev);
 }
 
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode) {

@@ -70,6 +70,14 @@ class Transformer:
     def forward(self, gen_token=True, use_graph=False, mode=SCHEDULE_FUSED):
         check(lib.awq_transformer_forward(self.h, int(gen_token), int(use_graph), mode))
 
+    def forward_logits(self, use_graph=False, mode=SCHEDULE_FUSED):
+        """run_llama_network() alone: this position's logits, no sampler."""
+        check(lib.awq_transformer_forward_logits(self.h, int(use_graph), mode))
+
+    def sample(self, sampler, gen_token=True):
+        """sample() (sampler.h:77-115) on this model's logits and token list."""
+        check(lib.awq_transformer_sample(self.h, sampler.h, int(gen_token)))
+
     def prefill(self, n_tokens, gen_token=True):
         """Consume n_tokens prompt tokens (already in the token list, from the current position) in one batched pass."""
         check(lib.awq_transformer_prefill(self.h, n_tokens, int(gen_token)))

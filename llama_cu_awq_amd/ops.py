@@ -181,6 +181,34 @@ def argmax_advance(ctx, logits, size, tokens, pos_host, pos_dev, write_token):
     check(lib.awq_argmax_advance(ctx.h, _addr(logits), size, _addr(tokens), _addr(pos_host), _addr(pos_dev), int(write_token)))
 
 
+def softmax_logits(ctx, logits, size, temperature):
+    """softmax_logits_kernel launch, sampler.h:87 (in place)."""
+    check(lib.awq_softmax_logits(ctx.h, _addr(logits), size, float(temperature)))
+
+
+def sample_top_p(ctx, probs, size, threshold, sorted_, tokens, pos_host, pos_dev):
+    """Sort + prefix sum + sample_top_p_kernel, sampler.h:94-115."""
+    check(lib.awq_sample_top_p(ctx.h, _addr(probs), size, float(threshold), int(sorted_), _addr(tokens), _addr(pos_host), _addr(pos_dev)))
+
+
+class Sampler:
+    """Sampler + build_sampler() / sample(), sampler.h:10-47, 77-115."""
+
+    def __init__(self, ctx, vocab_size, temperature, topp, rng_seed):
+        self.ctx = ctx
+        h = C.c_void_p()
+        check(lib.awq_sampler_create(ctx.h, vocab_size, float(temperature), float(topp), int(rng_seed), C.byref(h)))
+        self.h = h
+
+    def sample(self, logits, tokens, pos_host, pos_dev, gen_token):
+        check(lib.awq_sampler_sample(self.h, _addr(logits), _addr(tokens), _addr(pos_host), _addr(pos_dev), int(gen_token)))
+
+    def close(self):
+        if self.h:
+            check(lib.awq_sampler_destroy(self.h))
+            self.h = None
+
+
 def dequant(ctx, out, w, K, N):
     """(q - z) * scale materialised in fp16 (gpu_kernels.h:204-205)."""
     check(lib.awq_dequant(ctx.h, _addr(out), C.byref(w.c), K, N))

@@ -24,6 +24,12 @@
 //   attention                : fp64 softmax(qK^T/sqrt(d))V brute force
 //   argmax                   : brute force; ties -> lowest index (the
 //                              reference's tie winner is a write race)
+//   softmax of logits, top-p : fp64 softmax; numpy stable argsort + integer
+//                              cumulative sums; hand-built distributions whose
+//                              crossing index is known (the fp16 prefix sum of
+//                              the reference's CUB scan is order dependent:
+//                              "parity unpinned", the exact sum rounded once is
+//                              used instead)
 //   schedule / decode loop   : hand-traced toy model built from the above
 // The fp32 summation ORDER of the CUDA block/warp reductions comes from CUB,
 // which is not vendored in the reference: that order is "parity unpinned" and
@@ -428,6 +434,90 @@ int orc_argmax_advance(const uint16_t* logits, int size, int* tokens, int* pos_h
     *pos_host = p;
     if (pos_dev) *pos_dev = p;
     return best_i;
+}
+
+// ---------------------------------------------------------------- temperature / top-p sampling
+// xorshift* and the [0,1) float drawn from it (sampler.h:65-74).
+float orc_random_f32(unsigned long long* state) {
+    *state ^= *state >> 12;
+    *state ^= *state << 25;
+    *state ^= *state >> 27;
+    unsigned int r = (unsigned int)((*state * 0x2545F4914F6CDD1Dull) >> 32);
+    return (r >> 8) / 16777216.0f;
+}
+
+// softmax_logits_kernel (gpu_kernels.h:507-557), in place: l = half(l / T); v = expf(l - max) stored as half and
+// summed unrounded in fp32; p = half(float(half v) / sum).  The reference sums with cub::BlockReduce over 1024
+// threads (order unpinned); the order fixed here: thread t adds elements t, t+1024, ... in index order, the 1024
+// partials are then added as a balanced pairwise tree.
+void orc_softmax_logits(uint16_t* logits, int size, float temperature) {
+    for (int t = 0; t < size; t++) logits[t] = f2h(h2f(logits[t]) / temperature);
+    float max_val = -3.402823466e+38f;
+    for (int t = 0; t < size; t++) max_val = fmaxf(max_val, h2f(logits[t]));
+    float part[1024];
+    for (int t = 0; t < 1024; t++) part[t] = 0.0f;
+    for (int t = 0; t < 1024; t++)
+        for (int i = t; i < size; i += 1024) {
+            float v = expf(h2f(logits[i]) - max_val);
+            logits[i] = f2h(v);
+            part[t] += v;
+        }
+    for (int n = 1024; n > 1; n >>= 1)
+        for (int i = 0; i < n / 2; i++) part[i] = part[2 * i] + part[2 * i + 1];
+    const float sum = part[0];
+    for (int t = 0; t < size; t++) logits[t] = f2h(h2f(logits[t]) / sum);
+}
+
+// The reference's sort + inclusive prefix sum + sample_top_p_kernel (sampler.h:94-115, gpu_kernels.h:562-592),
+// written out step by step: sorted != 0 orders (probability, index) pairs by descending probability, stable (the
+// radix sort is); the prefix sum is exact (fp16 values are multiples of 2^-24, summed as integers) and rounded to fp16
+// once, where CUB's scan adds in fp16 in an order of its own ("parity unpinned"); the answer is the index at the first
+// position whose rounded prefix is >= threshold, position size-1 when none is.  Then the position advance of
+// gpu_kernels.h:582-591.  Returns the token.
+static uint64_t prob_units(uint16_t h) {
+    const uint32_t e = h >> 10, m = h & 0x3FFu;
+    return e == 0 ? (uint64_t)m : ((uint64_t)(m | 0x400u) << (e - 1));
+}
+int orc_sample_top_p(const uint16_t* probs, int size, float threshold, int sorted, int* tokens, int* pos_host, int* pos_dev) {
+    int* idx = (int*)malloc(sizeof(int) * (size_t)size);
+    for (int i = 0; i < size; i++) idx[i] = i;
+    if (sorted) {
+        // stable insertion-free sort: counting sort on the 16-bit key, descending, ties in index order
+        int* count = (int*)calloc(65537, sizeof(int));
+        for (int i = 0; i < size; i++) count[65535 - probs[i]]++;
+        int run = 0;
+        for (int k = 0; k < 65536; k++) { int c = count[k]; count[k] = run; run += c; }
+        for (int i = 0; i < size; i++) idx[count[65535 - probs[i]]++] = i;
+        free(count);
+    }
+    int pick = size - 1;
+    uint64_t run = 0;
+    for (int t = 0; t < size; t++) {
+        run += prob_units(probs[idx[t]]);
+        // exact value run * 2^-24 -> fp16 (one rounding, nearest even) -> float, as the kernel's (float)prefix[t]
+        const double exact = (double)run * 5.9604644775390625e-08;
+        const float rounded = h2f(f2h((float)exact));
+        // (float)exact is itself exact here only when run has <= 24 significant bits; round from the integer instead
+        float pref;
+        if (run < (1ull << 24)) {
+            pref = rounded;
+        } else {
+            const int e = 63 - __builtin_clzll(run);
+            const int shift = e - 10;
+            uint64_t mant = run >> shift;
+            const uint64_t rem = run & ((1ull << shift) - 1ull), half_ulp = 1ull << (shift - 1);
+            if (rem > half_ulp || (rem == half_ulp && (mant & 1ull))) mant++;
+            pref = ldexpf((float)mant, shift - 24);
+        }
+        if (pref >= threshold) { pick = t; break; }
+    }
+    const int token = idx[pick];
+    free(idx);
+    int p = *pos_host + 1;
+    tokens[p] = token;
+    *pos_host = p;
+    if (pos_dev) *pos_dev = p;
+    return token;
 }
 
 // ---------------------------------------------------------------- model image

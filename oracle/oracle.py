@@ -37,6 +37,9 @@ def _load():
         "orc_rope": ([vp, vp, i, i, i, vp, i, f], None),
         "orc_attention": ([vp, vp, vp, vp, vp, i, i, i, vp], None),
         "orc_argmax_advance": ([vp, i, vp, vp, vp, i], i),
+        "orc_random_f32": ([vp], f),
+        "orc_softmax_logits": ([vp, i, f], None),
+        "orc_sample_top_p": ([vp, i, f, i, vp, vp, vp], i),
         "orc_model_file_bytes": ([vp], C.c_size_t),
         "orc_model_open": ([vp, C.c_size_t], vp),
         "orc_model_close": ([vp], None),
@@ -137,6 +140,23 @@ def attention(q, key_cache, value_cache, num_heads, head_size, kv_mul, pos):
 def argmax_advance(logits, tokens, pos_host, pos_dev, write_token):
     ll = _c(logits.view(np.uint16), np.uint16)
     return lib.orc_argmax_advance(_p(ll), ll.size, _p(tokens), _p(pos_host), _p(pos_dev), int(write_token))
+
+
+def random_f32(state):
+    """state: np.uint64 array of 1 (updated in place). sampler.h:65-74."""
+    return float(lib.orc_random_f32(_p(state)))
+
+
+def softmax_logits(logits, temperature):
+    """Returns the fp16 probabilities (uint16 view in, new array out)."""
+    ll = np.array(logits.view(np.uint16), dtype=np.uint16, copy=True)
+    lib.orc_softmax_logits(_p(ll), ll.size, float(temperature))
+    return ll.view(np.float16)
+
+
+def sample_top_p(probs, threshold, sorted_, tokens, pos_host, pos_dev):
+    pp = _c(probs.view(np.uint16), np.uint16)
+    return lib.orc_sample_top_p(_p(pp), pp.size, float(threshold), int(sorted_), _p(tokens), _p(pos_host), _p(pos_dev))
 
 
 class Model:
