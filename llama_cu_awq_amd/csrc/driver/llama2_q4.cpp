@@ -43,6 +43,7 @@ static void error_usage(char* argv[]) {
     fprintf(stderr, "  -m <string> schedule: reference|fused|persistent, default fused\n");
     fprintf(stderr, "  -b <0|1>    consume the prompt in one batched prefill pass, default 0\n");
     fprintf(stderr, "  -e <0|1>    keep generating past the end-of-sequence token, default 0\n");
+    fprintf(stderr, "  -d <0|1>    print the GPU time of every token, default 0\n");
     exit(EXIT_FAILURE);
 }
 
@@ -77,6 +78,7 @@ int main(int argc, char* argv[]) {
     int steps = 0;
     std::string prompt;
     bool have_prompt = false;
+    int per_token_timings = 0;  // the reference's compile-time DUMP_PER_TOKEN_TIMINGS (llama2_q4.cu:32), as a switch
     float temperature = 0.5f;
     float topp = 0.6f;
     unsigned long long rng_seed = 0;
@@ -119,6 +121,7 @@ int main(int argc, char* argv[]) {
                 break;
             }
             case 'g': use_graph = atoi(argv[i + 1]); break;
+            case 'd': per_token_timings = atoi(argv[i + 1]); break;
             case 'e': ignore_eos = atoi(argv[i + 1]); break;
             case 'b': batched_prompt = atoi(argv[i + 1]); break;
             case 'm':
@@ -198,6 +201,12 @@ int main(int argc, char* argv[]) {
     while (pos < steps) {
         die_awq(awq_stream_sync(ctx));  // wait for the previous token, then launch the next before printing
         const bool gen_token = pos >= num_prompt_tokens - 1;
+        void *ev_start = nullptr, *ev_stop = nullptr;
+        if (per_token_timings) {  // llama2_q4.cu:545-550
+            die_awq(awq_event_create(ctx, &ev_start));
+            die_awq(awq_event_create(ctx, &ev_stop));
+            die_awq(awq_event_record(ctx, ev_start));
+        }
         if (temperature == 0.0f) {
             // network + greedy sampler as one (graph-replayed) unit; the coin the reference draws anyway is never used
             die_awq(awq_transformer_forward(t, gen_token, use_graph, mode));
@@ -205,6 +214,14 @@ int main(int argc, char* argv[]) {
             // run_transformer(), llama2_q4.cu:541-601: the network, then sample() (greedy while the prompt is consumed)
             die_awq(awq_transformer_forward_logits(t, use_graph, mode == AWQ_SCHEDULE_PERSISTENT ? AWQ_SCHEDULE_FUSED : mode));
             die_awq(awq_transformer_sample(t, sampler, gen_token));
+        }
+        if (per_token_timings) {  // llama2_q4.cu:592-600
+            float ms = 0.0f;
+            die_awq(awq_event_record(ctx, ev_stop));
+            die_awq(awq_event_elapsed_ms(ctx, ev_start, ev_stop, &ms));
+            printf(" t: %g ", ms);
+            die_awq(awq_event_destroy(ctx, ev_start));
+            die_awq(awq_event_destroy(ctx, ev_stop));
         }
         if (pos > 0) {
             next = st.shared_tokens[pos];
