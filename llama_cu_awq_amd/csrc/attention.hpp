@@ -11,7 +11,7 @@
 
 // Floats of LDS the function needs for a context of at most max_seq positions.
 __host__ __device__ constexpr int attention_head_lds_floats(int max_seq, int head_size, int waves) {
-    return ((max_seq + 3) & ~3) + waves * head_size + 2 * waves;
+    return ((max_seq + 3) & ~3) + waves * head_size;
 }
 
 // LP = lanes per position (head_size / 8), NW = waves of the calling workgroup (all of them must call).
@@ -21,10 +21,8 @@ template <int LP, int NW>
 __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att_head, const uint16_t* q_head,
                                                const uint16_t* k_head, const uint16_t* v_head, int head_size,
                                                int row_stride, float alpha, int size, float* lds) {
-    constexpr int T = NW * 64;
     float* sc = lds;                          // [size] scores (fp16-rounded values)
     float* acc_lds = lds + ((size + 3) & ~3);  // [NW][head_size]
-    float* red = acc_lds + NW * head_size;     // [2 * NW]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     constexpr int PW = 64 / LP;
     const int j = lane % LP, pr = lane / LP;
@@ -65,22 +63,15 @@ __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att
         }
     }
     __syncthreads();
+    // Softmax statistics: every wave computes them for itself from the scores in LDS, all in the same order (lane l
+    // takes positions l, l+64, ...; then the wave tree), so the values agree bit for bit and no further barrier or
+    // exchange is needed.
     float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed (its softmax block has 1024 threads)
-    for (int t = tid; t < size; t += T) m = fmaxf(m, sc[t]);
+    for (int t = lane; t < size; t += 64) m = fmaxf(m, sc[t]);
     m = wave_max(m);
-    if (lane == 0) red[wave] = m;
-    __syncthreads();
-    m = red[0];
-#pragma unroll
-    for (int w = 1; w < NW; w++) m = fmaxf(m, red[w]);
     float sum = 0.0f;
-    for (int t = tid; t < size; t += T) sum += expf(sc[t] - m);
+    for (int t = lane; t < size; t += 64) sum += expf(sc[t] - m);
     sum = wave_sum(sum);
-    if (lane == 0) red[NW + wave] = sum;
-    __syncthreads();
-    sum = 0.0f;
-#pragma unroll
-    for (int w = 0; w < NW; w++) sum += red[NW + w];
 
     float acc[8];
 #pragma unroll
