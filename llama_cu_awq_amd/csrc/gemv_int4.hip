@@ -284,11 +284,14 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     };
     auto issue = [&](Stage<NS>& st) {
         const int c = min(lp * 64 + lane, C - 1);  // lanes past the row end repeat its last chunk; consume() drops them
+        // byte offsets as unsigned 32-bit values on top of wave-uniform row pointers: the loads take the scalar-base
+        // form and need no 64-bit address arithmetic per lane
+        const uint32_t off_w = (uint32_t)c << 4, off_z = (uint32_t)(c >> 5) << 2, off_s = (uint32_t)(c >> 2) << 1;
 #pragma unroll
         for (int i = 0; i < NS; i++) {
-            st.w[i] = load_nt(reinterpret_cast<const u32x4*>(wrow[i]) + c);
-            st.zw[i] = zrow[i][c >> 5];
-            st.s[i] = srow[i][c >> 2];
+            st.w[i] = load_nt(reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(wrow[i]) + off_w));
+            st.zw[i] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(zrow[i]) + off_z);
+            st.s[i] = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(srow[i]) + off_s);
         }
         if (RES) {
 #pragma unroll
