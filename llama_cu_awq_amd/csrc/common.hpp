@@ -16,6 +16,12 @@ struct awq_ctx {
     // partial outputs and one arrival counter per head (self-resetting).
     float* attn_partial;
     unsigned int* attn_counter;
+    // Workspace of the prefill GEMM's split-K form (allocated on first use): fp32 partial tiles and per-tile arrival
+    // counters (self-resetting).
+    float* gemm_part;
+    size_t gemm_part_bytes;
+    unsigned int* gemm_counter;
+    size_t gemm_counter_count;
 };
 
 constexpr int kAttnMaxHeads = 256;

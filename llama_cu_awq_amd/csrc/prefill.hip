@@ -35,6 +35,9 @@ struct GemmParams {
     int C, pzh, sh;
     int epi;
     int mtiles, ntiles;
+    int ksplit;                  // 1, or 2: two workgroups share a tile, each taking half of K
+    float* part;                 // ksplit == 2: fp32 partial tiles [tile][2][128 x 128]
+    unsigned int* part_counter;  // ksplit == 2: arrivals per tile, zero between launches
     uint16_t* out[3];
     long long ldo[3];       // output row stride in elements
     long long out_off[3];   // element offset of output row 0 (KV cache: loff + pos0 * kv_dim)
@@ -145,9 +148,11 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int tile = (slot / p.mtiles) * 8 + xcd;
+    const int per_tile = p.mtiles * p.ksplit;
+    const int tile = (slot / per_tile) * 8 + xcd;
     if (tile >= p.ntiles) return;
-    const int m0 = (slot % p.mtiles) * BM;
+    const int m_index = (slot % per_tile) / p.ksplit, ks = (slot % per_tile) % p.ksplit;
+    const int m0 = m_index * BM;
 
     // activation loader: wave w, instruction q covers tile rows (4w + q) * 8 .. + 8 (8 lanes x 16 bytes per row);
     // the lane's LDS chunk is lane & 7, so it fetches the source chunk that the swizzle maps there
@@ -186,6 +191,10 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
 
     const int nsteps = (p.K + BK - 1) / BK;
     const int k_last = (nsteps - 1) * BK;
+    // split K: the halves meet at an even step, so that both start on a quantisation group
+    const int s_split = (nsteps / 2) & ~1;
+    const int s_begin = ks ? s_split : 0;
+    const int s_end = (p.ksplit == 2 && ks == 0) ? s_split : nsteps;
     auto load_a = [&](int step) {  // 4 loads
         const int k0 = min(step * BK, k_last);
         const uint32_t dst = (uint32_t)((step % A_STAGES) * TILE_BYTES + wave * 4096);
@@ -228,14 +237,14 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
         }
     };
 
-    // Prologue: activation tiles 0, 1 and weight pairs 0, 1.
-    load_a(0);
-    load_a(1);
-    load_w(0);
-    load_w(1);
+    // Prologue: the first two activation tiles and weight pairs.
+    load_a(s_begin);
+    load_a(s_begin + 1);
+    load_w(s_begin >> 1);
+    load_w((s_begin >> 1) + 1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    for (int step = 0; step < nsteps; step += 2) {
+    for (int step = s_begin; step < s_end; step += 2) {
         // even step: request activation tile step+2 and weight pair (step/2)+2, then multiply
         load_a(step + 2);  // into the slot that step-1 multiplied: every wave is past the barrier that ended it
         load_w((step >> 1) + 2);  // into the slot this wave finished reading at the end of the previous iteration
@@ -249,6 +258,34 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
         // needed next: activation tile step+2 (followed by 4 + 4 loads) and weight pair (step/2)+1 (older still)
         asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         __syncthreads();
+    }
+
+    if (p.ksplit == 2) {
+        // The two halves of K meet here.  Each workgroup writes its fp32 partial tile through to memory and counts
+        // itself in; the first to arrive leaves, the second adds the other's partial to its own (a two-term fp32 sum
+        // does not depend on which one that is) and goes on to the epilogue.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no direct-to-LDS load is still on its way
+        __syncthreads();
+        const size_t tile_id = (size_t)tile * p.mtiles + m_index;
+        float* mine = p.part + (tile_id * 2 + ks) * (size_t)(BM * BN);
+        const float* other = p.part + (tile_id * 2 + (ks ^ 1)) * (size_t)(BM * BN);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 16; j++)
+                __hip_atomic_store(&mine[((wave * 4 + i) * 16 + j) * 64 + lane], acc[i][j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        unsigned int* arrival = reinterpret_cast<unsigned int*>(lds_bytes);
+        if (tid == 0) *arrival = __hip_atomic_fetch_add(&p.part_counter[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*arrival == 0u) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        if (tid == 0) p.part_counter[tile_id] = 0;  // ready for the next launch
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 16; j++) acc[i][j] += other[((wave * 4 + i) * 16 + j) * 64 + lane];
     }
 
     // epilogue: acc[i][j] is D[row = 32*i + 8*(j/4) + 4*(lane/32) + j%4][col = lane%32] of the wave's 32 columns
@@ -603,8 +640,31 @@ static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* 
     }
     p.mtiles = div_up(p.M, pf::BM);
     p.ntiles = ntiles;
-    // ids go round-robin over the 8 XCDs; each XCD takes every 8th weight tile with all of its M tiles
-    const int grid = 8 * p.mtiles * div_up(ntiles, 8);
+    p.ksplit = 1;
+    // A single matrix with fewer tiles than compute units: two workgroups per tile, each half of K.
+    if ((p.epi == pf::EPI_STORE || p.epi == pf::EPI_RESID) && p.mtiles * ntiles < 256 && p.K >= 8 * pf::BK) {
+        const size_t tiles = (size_t)p.mtiles * ntiles;
+        const size_t need = tiles * 2 * pf::BM * pf::BN * sizeof(float);
+        if (ctx->gemm_part_bytes < need || ctx->gemm_counter_count < tiles) {
+            AWQ_HIP_TRY(hipStreamSynchronize(ctx->stream));
+            if (ctx->gemm_part) (void)hipFree(ctx->gemm_part);
+            if (ctx->gemm_counter) (void)hipFree(ctx->gemm_counter);
+            ctx->gemm_part = nullptr;
+            ctx->gemm_counter = nullptr;
+            ctx->gemm_part_bytes = 0;
+            ctx->gemm_counter_count = 0;
+            AWQ_HIP_TRY(hipMalloc((void**)&ctx->gemm_part, need));
+            AWQ_HIP_TRY(hipMalloc((void**)&ctx->gemm_counter, tiles * sizeof(unsigned int)));
+            AWQ_HIP_TRY(hipMemset(ctx->gemm_counter, 0, tiles * sizeof(unsigned int)));
+            ctx->gemm_part_bytes = need;
+            ctx->gemm_counter_count = tiles;
+        }
+        p.ksplit = 2;
+        p.part = ctx->gemm_part;
+        p.part_counter = ctx->gemm_counter;
+    }
+    // ids go round-robin over the 8 XCDs; each XCD takes every 8th weight tile with all of its M tiles (and K halves)
+    const int grid = 8 * p.mtiles * p.ksplit * div_up(ntiles, 8);
     hipLaunchKernelGGL(pf::gemm_int4_kernel, dim3(grid), dim3(256), pf::GEMM_LDS_BYTES, ctx->stream, p);
     return awq_check_launch(what);
 }

@@ -58,6 +58,10 @@ static int ctx_init(int device, hipStream_t stream, bool owns, awq_ctx** out) {
     c->owns_stream = owns;
     c->attn_partial = nullptr;
     c->attn_counter = nullptr;
+    c->gemm_part = nullptr;
+    c->gemm_part_bytes = 0;
+    c->gemm_counter = nullptr;
+    c->gemm_counter_count = 0;
     size_t partial_bytes = (size_t)kAttnMaxHeads * kAttnMaxSplits * kAttnMaxHeadSize * sizeof(float);
     hipError_t e = hipMalloc((void**)&c->attn_partial, partial_bytes);
     if (e == hipSuccess) e = hipMalloc((void**)&c->attn_counter, kAttnMaxHeads * sizeof(unsigned int));
@@ -96,6 +100,8 @@ int awq_ctx_destroy(awq_ctx* ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->attn_partial);
     (void)hipFree(ctx->attn_counter);
+    if (ctx->gemm_part) (void)hipFree(ctx->gemm_part);
+    if (ctx->gemm_counter) (void)hipFree(ctx->gemm_counter);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return AWQ_OK;
