@@ -354,17 +354,50 @@ __global__ __launch_bounds__(256) void embed_rows_kernel(uint16_t* x, const uint
     for (int i = threadIdx.x; i < (dim >> 3); i += 256) dst[i] = src[i];
 }
 
-// o[m] = half(x[m] * (rsqrt(mean(x[m]^2) + 1e-5) * w))  (gpu_kernels.h:72-105, one workgroup per token row)
+// o[m] = half(x[m] * (rsqrt(mean(x[m]^2) + 1e-5) * w))  (gpu_kernels.h:72-105, one workgroup per token row).
+// 16-byte pieces; up to 4 per thread stay in registers between the two passes (rows of up to 8192), longer rows
+// re-read the rest.
 __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(uint16_t* o, const uint16_t* x, const uint16_t* weight, int size) {
     __shared__ float red[4];
+    constexpr int NP = 4;
     const int tid = threadIdx.x;
-    const uint16_t* xr = x + (size_t)blockIdx.x * size;
-    uint16_t* orow = o + (size_t)blockIdx.x * size;
-    float part = 0.0f;
-    for (int i = tid; i < size; i += 256) {
-        const float v = half_bits_to_float(xr[i]);
-        part = fmaf(v, v, part);
+    const int n8 = size >> 3;
+    const u32x4* xr = reinterpret_cast<const u32x4*>(x + (size_t)blockIdx.x * size);
+    const u32x4* wr = reinterpret_cast<const u32x4*>(weight);
+    u32x4* orow = reinterpret_cast<u32x4*>(o + (size_t)blockIdx.x * size);
+    u32x4 v[NP], w[NP];
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+        const int e = min(i * 256 + tid, n8 - 1);
+        v[i] = xr[e];
+        w[i] = wr[e];
     }
+    auto sumsq = [](const u32x4 p, float part) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const h16x2 h = as_h2(p[k]);
+            part = fmaf((float)h[0], (float)h[0], part);
+            part = fmaf((float)h[1], (float)h[1], part);
+        }
+        return part;
+    };
+    auto scale = [](const u32x4 p, const u32x4 wv, float ss) {
+        u32x4 r;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const h16x2 h = as_h2(p[k]), hw = as_h2(wv[k]);
+            h16x2 q;
+            q[0] = (h16_t)((float)h[0] * (ss * (float)hw[0]));
+            q[1] = (h16_t)((float)h[1] * (ss * (float)hw[1]));
+            r[k] = as_u32(q);
+        }
+        return r;
+    };
+    float part = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NP; i++)
+        if (i * 256 + tid < n8) part = sumsq(v[i], part);
+    for (int e = NP * 256 + tid; e < n8; e += 256) part = sumsq(xr[e], part);
     part = wave_sum(part);
     if ((tid & 63) == 0) red[tid >> 6] = part;
     __syncthreads();
@@ -372,22 +405,32 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(uint16_t* o, const ui
     ss /= (float)size;
     ss += 1e-5f;
     ss = 1.0f / sqrtf(ss);
-    for (int i = tid; i < size; i += 256) orow[i] = float_to_half_bits(half_bits_to_float(xr[i]) * (ss * half_bits_to_float(weight[i])));
+#pragma unroll
+    for (int i = 0; i < NP; i++)
+        if (i * 256 + tid < n8) orow[i * 256 + tid] = scale(v[i], w[i], ss);
+    for (int e = NP * 256 + tid; e < n8; e += 256) orow[e] = scale(xr[e], wr[e], ss);
 }
 
 // RoPE of q rows [M][heads*hs] and of the K cache rows pos0..pos0+M-1 (gpu_kernels.h:340-363 per position).
 __global__ void rope_rows_kernel(uint16_t* q, uint16_t* kcache_layer, int num_heads, int num_kv_heads, int head_size, int pos0,
-                                 float rope_theta) {
+                                 float rope_theta, const float2* table) {
     const int m = blockIdx.y;
     const int h = blockIdx.x;
     const int i = threadIdx.x;
     const int pos = pos0 + m;
     const int half_size = head_size >> 1;
-    const int head_dim = (i * 2) % head_size;
-    const float freq = 1.0f / powf(rope_theta, head_dim / (float)head_size);
-    const float val = pos * freq;
-    const float fcr = cosf(val);
-    const float fci = sinf(val);
+    float fcr, fci;
+    if (table) {  // (cos, sin) per position and pair, computed once at load time with the formula below
+        const float2 cs = table[(size_t)pos * half_size + i];
+        fcr = cs.x;
+        fci = cs.y;
+    } else {
+        const int head_dim = (i * 2) % head_size;
+        const float freq = 1.0f / powf(rope_theta, head_dim / (float)head_size);
+        const float val = pos * freq;
+        fcr = cosf(val);
+        fci = sinf(val);
+    }
     uint16_t* qh = q + ((size_t)m * num_heads + h) * head_size;
     const float q0 = half_bits_to_float(qh[i]);
     const float q1 = half_bits_to_float(qh[i + half_size]);
@@ -729,8 +772,10 @@ int awq_launch_rmsnorm_rows(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const 
     return awq_check_launch("rmsnorm_rows");
 }
 
-int awq_launch_rope_rows(awq_ctx* ctx, uint16_t* q, uint16_t* kcache_layer, int nh, int nkv, int hs, int pos0, float theta, int M) {
-    hipLaunchKernelGGL(pf::rope_rows_kernel, dim3(nh, M), dim3(hs / 2), 0, ctx->stream, q, kcache_layer, nh, nkv, hs, pos0, theta);
+int awq_launch_rope_rows(awq_ctx* ctx, uint16_t* q, uint16_t* kcache_layer, int nh, int nkv, int hs, int pos0, float theta, int M,
+                         const float2* table) {
+    hipLaunchKernelGGL(pf::rope_rows_kernel, dim3(nh, M), dim3(hs / 2), 0, ctx->stream, q, kcache_layer, nh, nkv, hs, pos0, theta,
+                       table);
     return awq_check_launch("rope_rows");
 }
 

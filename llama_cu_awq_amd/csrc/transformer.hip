@@ -38,7 +38,8 @@ int awq_launch_gemm_ffn(awq_ctx* ctx, uint16_t* hb, const uint16_t* A, int lda, 
                         const awq_qweight* up_w, int K, int N);
 int awq_launch_embed_rows(awq_ctx* ctx, uint16_t* x, const uint16_t* table, int dim, const int* tokens, int pos0, int M);
 int awq_launch_rmsnorm_rows(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const uint16_t* w, int size, int M);
-int awq_launch_rope_rows(awq_ctx* ctx, uint16_t* q, uint16_t* kcache_layer, int nh, int nkv, int hs, int pos0, float theta, int M);
+int awq_launch_rope_rows(awq_ctx* ctx, uint16_t* q, uint16_t* kcache_layer, int nh, int nkv, int hs, int pos0, float theta, int M,
+                         const float2* table);
 int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, const uint16_t* kc, const uint16_t* vc, int nh, int hs,
                             int kv_mul, int M, int pos0);
 int awq_launch_set_pos(awq_ctx* ctx, int* pos_dev, volatile int* pos_host, int value);
@@ -735,7 +736,8 @@ int awq_transformer_prefill(awq_transformer* t, int n_tokens, int gen_token) {
             if ((r = awq_launch_gemm_qkv(ctx, t->pf_q, t->s.key_cache, t->s.value_cache, loff + (long long)pos0 * kv_dim, t->pf_xb,
                                          dim, M, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, kv_dim)))
                 return r;
-            if ((r = awq_launch_rope_rows(ctx, t->pf_q, t->s.key_cache + loff, p.n_heads, p.n_kv_heads, hs, pos0, p.rope_theta, M)))
+            if ((r = awq_launch_rope_rows(ctx, t->pf_q, t->s.key_cache + loff, p.n_heads, p.n_kv_heads, hs, pos0, p.rope_theta, M,
+                                          t->rope_table)))
                 return r;
             if ((r = awq_launch_attn_prefill(ctx, t->pf_att, t->pf_q, t->s.key_cache + loff, t->s.value_cache + loff, p.n_heads, hs,
                                              kv_mul, M, pos0)))
