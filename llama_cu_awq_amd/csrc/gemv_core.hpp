@@ -1,0 +1,182 @@
+// Device-side building blocks of the int4 matrix-vector kernels (gemv_int4.hip): the dequantise-and-dot of one
+// 32-element chunk, the register image of one 64-lane pass, and the staging of the activation vector into LDS.
+#pragma once
+
+#include "common.hpp"
+
+namespace gemv {
+
+// What staging needs to know about the activation vector.
+struct XArgs {
+    const uint16_t* x;       // K halves
+    const uint16_t* norm_w;  // RMSNorm weights (NORM forms)
+    uint16_t* norm_out;      // optional: workgroup (0, 0) also stores the normalised vector here
+    int K;
+    int C;                   // 32-element chunks = ceil(K / 32)
+};
+
+// sum over the 32 consecutive K elements of one chunk of (q - z) * x.
+//
+// w: 4 dwords of 8 nibbles.  xq[qi]: the 8 activations of dword qi as fp16 pairs
+// (x0,x4) (x1/16,x5/16) (x2,x6) (x3/16,x7/16).  OR-ing a nibble into the
+// mantissa of fp16 1024.0 gives 1024+q (nibble at bits 0-3) or 1024+16q (bits
+// 4-7) exactly, so
+//   sum_k (1024 + [16] q_k) * X_k  =  1024 * sum_k X_k  +  sum_k q_k x_k
+// and the chunk's constants A = sum x and B = 1024 * sum X (computed once when
+// x is staged) turn that into sum (q - z) x = dot - B - z*A.  The accumulator
+// starts at -B - z*A so that the large common term cancels first.  Products are
+// exact in fp32 (11-bit x 11-bit significands); only the fp32 additions round.
+__device__ __forceinline__ float chunk_dot(const u32x4 w, const float zf, const u32x4 (&xq)[4], const float A, const float B,
+                                           const uint32_t magic) {
+    float acc = fmaf(-zf, A, -B);
+#pragma unroll
+    for (int qi = 0; qi < 4; qi++) {
+        const uint32_t d = w[qi];
+        const uint32_t d8 = d >> 8;
+        acc = dot2((d & 0x000F000Fu) | magic, xq[qi][0], acc);
+        acc = dot2((d & 0x00F000F0u) | magic, xq[qi][1], acc);
+        acc = dot2((d8 & 0x000F000Fu) | magic, xq[qi][2], acc);
+        acc = dot2((d8 & 0x00F000F0u) | magic, xq[qi][3], acc);
+    }
+    return acc;
+}
+
+// One 64-lane pass over the NS row streams of a wave: 16 bytes of packed weights per lane and stream, the zero-point
+// dword and the scale that cover them, and (residual form) the value the result is added to.
+template <int NS>
+struct Stage {
+    u32x4 w[NS];
+    uint32_t zw[NS];
+    uint16_t s[NS];
+    uint16_t res[NS];
+};
+
+// Staging of x (K halves) into LDS: xs[qi*C + c] holds the 8 activations of dword qi of chunk c as pairs
+// (x0,x4)(x1/16,x5/16)(x2,x6)(x3/16,x7/16), and ab[c] = {A, B} the chunk constants described at chunk_dot.  Elements
+// in [K, 32*C) are zero.  With NORM the vector is RMS-normalised on the way in with the reference's arithmetic
+// (gpu_kernels.h:72-105): o = half(x * (rsqrt(mean(x^2) + 1e-5) * w)).
+//
+// Loads return in order, so the activations are requested (load_x) before the first stages of packed weights and
+// staged (stage_x) while those are still on their way: XP pieces of 8 halves per thread travel in registers, the rest
+// of a longer vector is fetched late by stage_x itself.
+constexpr int XP = 2;
+
+template <bool NORM>
+struct XPieces {
+    u32x4 v[XP];
+    u32x4 w[NORM ? XP : 1];
+};
+
+template <int W, bool NORM>
+__device__ __forceinline__ void load_x(XPieces<NORM>& xr, const XArgs& p) {
+    constexpr int T = W * 64;
+    const int n8 = p.K >> 3;  // 8-half pieces of real data
+    const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
+    const u32x4* wg = reinterpret_cast<const u32x4*>(p.norm_w);
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        const int e = min(i * T + (int)threadIdx.x, n8 - 1);  // clamped, masked in stage_x
+        xr.v[i] = xg[e];
+        if (NORM) xr.w[i] = wg[e];
+    }
+}
+
+// One piece of 8 halves: normalise (optional), permute, reduce the chunk constants over the 4 lanes of a chunk, store.
+template <bool NORM>
+__device__ __forceinline__ void stage_piece(u32x4* xs, float2* ab, const XArgs& p, int e, u32x4 v, u32x4 wv, float ss,
+                                            bool store_norm) {
+    const int n8 = p.K >> 3;
+    if (e >= n8) v = u32x4{0u, 0u, 0u, 0u};
+    if (NORM) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const h16x2 h = as_h2(v[i]);
+            const h16x2 hw = as_h2(wv[i]);
+            h16x2 o;
+            o[0] = (h16_t)((float)h[0] * (ss * (float)hw[0]));
+            o[1] = (h16_t)((float)h[1] * (ss * (float)hw[1]));
+            v[i] = as_u32(o);
+        }
+        if (store_norm && e < n8) reinterpret_cast<u32x4*>(p.norm_out)[e] = v;
+    }
+    const h16x2 sixteenth = {(h16_t)0.0625f, (h16_t)0.0625f};
+    // v holds halves h0..h7 as (h0,h1)(h2,h3)(h4,h5)(h6,h7) -> (h0,h4)(h1,h5)(h2,h6)(h3,h7)
+    const h16x2 p0 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x05040100u));
+    const h16x2 p1 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x07060302u)) * sixteenth;
+    const h16x2 p2 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x05040100u));
+    const h16x2 p3 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x07060302u)) * sixteenth;
+    // fp32 sums of the stored halves: dot products against (1, 1)
+    const uint32_t ones = 0x3C003C00u;
+    const float even = dot2(as_u32(p0), ones, dot2(as_u32(p2), ones, 0.0f));
+    const float odd = dot2(as_u32(p1), ones, dot2(as_u32(p3), ones, 0.0f));
+    float a = fmaf(16.0f, odd, even);  // sum of the activations as the dot product sees them
+    float b = even + odd;              // sum of the stored fp16 values
+    // the 4 dword pieces of a chunk sit in 4 adjacent lanes
+    a += dpp_mov<0xB1>(a);
+    a += dpp_mov<0x4E>(a);
+    b += dpp_mov<0xB1>(b);
+    b += dpp_mov<0x4E>(b);
+    if (e < p.C * 4) {
+        u32x4 o = {as_u32(p0), as_u32(p1), as_u32(p2), as_u32(p3)};
+        xs[(e & 3) * p.C + (e >> 2)] = o;
+        if ((e & 3) == 0) ab[e >> 2] = make_float2(a, 1024.0f * b);
+    }
+}
+
+__device__ __forceinline__ float piece_sumsq(u32x4 v, float part) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const h16x2 h = as_h2(v[i]);
+        const float a = (float)h[0], b = (float)h[1];
+        part = fmaf(a, a, part);
+        part = fmaf(b, b, part);
+    }
+    return part;
+}
+
+template <int W, bool NORM>
+__device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const XArgs& p, float* red, const XPieces<NORM>& xr) {
+    constexpr int T = W * 64;
+    const int tid = threadIdx.x;
+    const int n8 = p.K >> 3;
+    const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
+    const u32x4* wg = reinterpret_cast<const u32x4*>(p.norm_w);
+    float ss = 0.0f;
+    if (NORM) {
+        float part = 0.0f;
+#pragma unroll
+        for (int i = 0; i < XP; i++)
+            if (i * T + tid < n8) part = piece_sumsq(xr.v[i], part);
+        for (int e = XP * T + tid; e < n8; e += T) part = piece_sumsq(xg[e], part);
+        part = wave_sum(part);
+        if ((tid & 63) == 0) red[tid >> 6] = part;
+        __syncthreads();
+        float r[W];
+#pragma unroll
+        for (int i = 0; i < W; i++) r[i] = red[i];
+#pragma unroll
+        for (int n = W; n > 1; n >>= 1)
+#pragma unroll
+            for (int i = 0; i < n / 2; i++) r[i] = r[2 * i] + r[2 * i + 1];
+        ss = r[0];
+        ss /= (float)p.K;
+        ss += 1e-5f;
+        ss = 1.0f / sqrtf(ss);
+    }
+    const bool store_norm = NORM && p.norm_out != nullptr && blockIdx.x == 0 && blockIdx.y == 0;
+#pragma unroll
+    for (int i = 0; i < XP; i++)
+        if (i * T < p.C * 4)  // uniform: the quad reduction needs all lanes
+            stage_piece<NORM>(xs, ab, p, i * T + tid, xr.v[i], xr.w[NORM ? i : 0], ss, store_norm);
+    for (int e0 = XP * T; e0 < p.C * 4; e0 += T) {
+        const int e = e0 + tid;
+        const int ec = min(e, n8 - 1);
+        const u32x4 v = xg[ec];
+        u32x4 wv = v;
+        if (NORM) wv = wg[ec];
+        stage_piece<NORM>(xs, ab, p, e, v, wv, ss, store_norm);
+    }
+    __syncthreads();
+}
+
+}  // namespace gemv
