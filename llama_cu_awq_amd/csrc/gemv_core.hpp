@@ -75,6 +75,7 @@ __device__ __forceinline__ void load_x(XPieces<NORM>& xr, const XArgs& p) {
     const u32x4* wg = reinterpret_cast<const u32x4*>(p.norm_w);
 #pragma unroll
     for (int i = 0; i < XP; i++) {
+        if (i > 0 && i * T >= n8) break;  // uniform: nothing left for this piece
         const int e = min(i * T + (int)threadIdx.x, n8 - 1);  // clamped, masked in stage_x
         xr.v[i] = xg[e];
         if (NORM) xr.w[i] = wg[e];
@@ -88,13 +89,17 @@ __device__ __forceinline__ void stage_piece(u32x4* xs, float2* ab, const XArgs& 
     const int n8 = p.K >> 3;
     if (e >= n8) v = u32x4{0u, 0u, 0u, 0u};
     if (NORM) {
+        // (float)h * f as fma(h, f, -0): exact, and the fp16 -> fp32 conversion rides in the multiply (v_fma_mix_f32);
+        // the addend sits in a register the compiler cannot see through, or it would fold the fma away again
+        float nz = -0.0f;
+        asm("" : "+v"(nz));
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const h16x2 h = as_h2(v[i]);
             const h16x2 hw = as_h2(wv[i]);
             h16x2 o;
-            o[0] = (h16_t)((float)h[0] * (ss * (float)hw[0]));
-            o[1] = (h16_t)((float)h[1] * (ss * (float)hw[1]));
+            o[0] = (h16_t)__builtin_fmaf((float)h[0], __builtin_fmaf((float)hw[0], ss, nz), nz);
+            o[1] = (h16_t)__builtin_fmaf((float)h[1], __builtin_fmaf((float)hw[1], ss, nz), nz);
             v[i] = as_u32(o);
         }
         if (store_norm && e < n8) reinterpret_cast<u32x4*>(p.norm_out)[e] = v;
@@ -134,6 +139,7 @@ __device__ __forceinline__ float piece_sumsq(u32x4 v, float part) {
     return part;
 }
 
+// red: W + 1 floats of LDS.
 template <int W, bool NORM>
 __device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const XArgs& p, float* red, const XPieces<NORM>& xr) {
     constexpr int T = W * 64;
@@ -151,17 +157,24 @@ __device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const XArgs& p, f
         part = wave_sum(part);
         if ((tid & 63) == 0) red[tid >> 6] = part;
         __syncthreads();
-        float r[W];
+        // the correctly rounded divide, square root and reciprocal are ~60 instructions on a uniform value: one wave
+        // computes them for the workgroup
+        if (tid < 64) {
+            float r[W];
 #pragma unroll
-        for (int i = 0; i < W; i++) r[i] = red[i];
+            for (int i = 0; i < W; i++) r[i] = red[i];
 #pragma unroll
-        for (int n = W; n > 1; n >>= 1)
+            for (int n = W; n > 1; n >>= 1)
 #pragma unroll
-            for (int i = 0; i < n / 2; i++) r[i] = r[2 * i] + r[2 * i + 1];
-        ss = r[0];
-        ss /= (float)p.K;
-        ss += 1e-5f;
-        ss = 1.0f / sqrtf(ss);
+                for (int i = 0; i < n / 2; i++) r[i] = r[2 * i] + r[2 * i + 1];
+            float t = r[0];
+            t /= (float)p.K;
+            t += 1e-5f;
+            t = 1.0f / sqrtf(t);
+            if (tid == 0) red[W] = t;
+        }
+        __syncthreads();
+        ss = red[W];
     }
     const bool store_norm = NORM && p.norm_out != nullptr && blockIdx.x == 0 && blockIdx.y == 0;
 #pragma unroll
