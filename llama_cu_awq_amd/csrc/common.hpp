@@ -25,7 +25,7 @@ struct awq_ctx {
 };
 
 constexpr int kAttnMaxHeads = 256;
-constexpr int kAttnMaxSplits = 32;
+constexpr int kAttnMaxSplits = 16;
 constexpr int kAttnMaxHeadSize = 256;
 constexpr int kAttnFusedMaxSeq = 512;  // up to this launch size attention runs as one workgroup per head
 

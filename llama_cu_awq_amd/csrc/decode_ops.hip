@@ -469,7 +469,9 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
     hipLaunchKernelGGL((attn_scores_kernel<LP>), dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, ctx->stream, att, q,
                        key_cache, head_size, kv_mul, row_stride, alpha, pos);
     if (int r = awq_check_launch("attn_scores")) return r;
-    int nsplit = div_up(max_seq_len, 64);  // one round of value rows per workgroup
+    // one or two rounds of value rows per workgroup; more than 16 splits cost more in the exchange of partial sums
+    // (same-address arrivals, partials to add) than the extra workgroups bring
+    int nsplit = div_up(max_seq_len, 128);
     if (nsplit > kAttnMaxSplits) nsplit = kAttnMaxSplits;
     if (nsplit < 1) nsplit = 1;
     hipLaunchKernelGGL((attn_softmax_pv_kernel<LP>), dim3(nsplit, num_heads), dim3(256), 0, ctx->stream, output, att,

@@ -361,12 +361,8 @@ int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan
     static const int forced_r = env_int("AWQ_GEMV_ROWS");
     static const int forced_d = env_int("AWQ_GEMV_DEPTH");
     static const int forced_g = env_int("AWQ_GEMV_GROUPS_PER_WG");
-    static const int forced_nw = env_int("AWQ_GEMV_NORM_WAVES");
-    static const int forced_nr = env_int("AWQ_GEMV_NORM_ROWS");
     if (forced_w) plan.waves = forced_w;
     if (forced_r) plan.rows = forced_r;
-    if (p.norm_w && forced_nw) plan.waves = forced_nw;
-    if (p.norm_w && forced_nr) plan.rows = forced_nr;
     if (forced_d) plan.depth = forced_d;
     if (forced_g) plan.groups = forced_g;
     if (ROPE && plan.rows < 2) plan.rows = 2;  // a rotation pair lives in one wave
