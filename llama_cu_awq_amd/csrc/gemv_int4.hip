@@ -44,7 +44,6 @@ struct GemvParams {
     float inv_gpu_count;
     int loff[3];             // -1: none; else out += loff + *pos * N
     const int* pos;
-    int groups_per_wg;       // row groups (4 waves x R rows) a workgroup walks through
     const float2* rope;      // fused RoPE: (cos, sin) table [position][head_size/2], or null
     int head_size;           // for the fused RoPE row pairing
 };
@@ -90,10 +89,10 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     // then pass); D stages are in flight at any time.  The sequence is padded to a multiple of D with repeats of the
     // last stage, which are loaded (same addresses again) but not accumulated, so that the number of loads between a
     // stage's request and its use is a compile-time constant.
+    // The workgroup takes row groups blockIdx.x, blockIdx.x + gridDim.x, ... (x is staged once for all of them).
     const int groups_total = (p.N + W * R - 1) / (W * R);
-    const int g_begin = blockIdx.x * p.groups_per_wg;
-    const int g_end = min(groups_total, g_begin + p.groups_per_wg);
-    const int total = (g_end - g_begin) * P;
+    const int g_begin = blockIdx.x, g_stride = gridDim.x;
+    const int total = ((groups_total - 1 - g_begin) / g_stride + 1) * P;
 
     // ---- load cursor
     const uint32_t* wrow[NS];
@@ -141,7 +140,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
             lp++;
             if (lp == P) {
                 lp = 0;
-                lg++;
+                lg += g_stride;
                 set_rows(lg);
             }
         }
@@ -218,7 +217,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
             if (cp == P) {
                 finish_group(st);
                 cp = 0;
-                cg++;
+                cg += g_stride;
             }
         }
     };
@@ -294,7 +293,6 @@ void fill_common(GemvParams& p, const uint16_t* x, int K, int N) {
     p.inv_gpu_count = 1.0f;
     p.loff[0] = p.loff[1] = p.loff[2] = -1;
     p.pos = nullptr;
-    p.groups_per_wg = 1;
     p.rope = nullptr;
     p.head_size = 0;
 }
@@ -303,19 +301,38 @@ Int4Mat to_mat(const awq_qweight* w) { return Int4Mat{w->weight, w->zeros, w->sc
 
 bool qw_ok(const awq_qweight* w) { return w && w->weight && w->zeros && w->scales; }
 
+// Tuning overrides for experiments: AWQ_GEMV_WAVES, AWQ_GEMV_ROWS, AWQ_GEMV_DEPTH.
+int env_int(const char* name) {
+    const char* e = getenv(name);
+    return e ? atoi(e) : 0;
+}
+
 // Launch geometry of one matrix-vector product.
 struct GemvPlan {
     int waves;   // waves per workgroup (4, 8)
     int rows;    // rows per wave (1, 2, 4)
     int depth;   // stages in flight per wave (2, 3, 4)
-    int groups;  // row groups per workgroup
 };
 
 template <int W, int R, int D, int KIND, bool ROPE>
-int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, int groups_per_wg) {
+int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     const int groups_total = div_up(p.N, W * R);
-    p.groups_per_wg = groups_per_wg;
-    const dim3 grid(div_up(groups_total, p.groups_per_wg), grid_y);
+    int gx = groups_total;
+    // The norm-fused gate/up kernel stages (and normalises) x in every workgroup, and that work is what bounds it:
+    // two workgroups per compute unit walk the row groups between them (measured best at the 7B shape; the plain
+    // kernels are faster with one group per workgroup).
+    if (p.norm_w && KIND == KIND_FFN) {
+        static int cus = 0;
+        if (!cus) {
+            int dev = 0, n = 0;
+            if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+                cus = n;
+            else
+                cus = 256;
+        }
+        if (gx > 2 * cus) gx = 2 * cus;
+    }
+    const dim3 grid(gx, grid_y);
     const size_t lds = (size_t)p.C * 72;  // activations + per-chunk constants
     if (p.norm_w)
         hipLaunchKernelGGL((gemv_int4_kernel<W, R, D, KIND, true, ROPE>), grid, dim3(W * 64), lds, ctx->stream, p);
@@ -330,19 +347,14 @@ int dispatch_depth(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, co
     int depth = plan.depth;
     while (depth > 2 && (NS * depth > 16 || depth > 4)) depth--;  // what the register file affords
     switch (depth) {
-        case 2: return launch<W, R, 2, KIND, ROPE>(ctx, p, grid_y, what, plan.groups);
-        case 3: if constexpr (NS * 3 <= 16) return launch<W, R, 3, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
-        case 4: if constexpr (NS * 4 <= 16) return launch<W, R, 4, KIND, ROPE>(ctx, p, grid_y, what, plan.groups); break;
+        case 2: return launch<W, R, 2, KIND, ROPE>(ctx, p, grid_y, what);
+        case 3: if constexpr (NS * 3 <= 16) return launch<W, R, 3, KIND, ROPE>(ctx, p, grid_y, what); break;
+        case 4: if constexpr (NS * 4 <= 16) return launch<W, R, 4, KIND, ROPE>(ctx, p, grid_y, what); break;
     }
     awq_set_error("no int4 matrix-vector kernel with %d stages in flight for %d streams", plan.depth, NS);
     return AWQ_ERR_ARG;
 }
 
-// Tuning overrides for experiments: AWQ_GEMV_WAVES, AWQ_GEMV_ROWS, AWQ_GEMV_DEPTH, AWQ_GEMV_GROUPS_PER_WG.
-int env_int(const char* name) {
-    const char* e = getenv(name);
-    return e ? atoi(e) : 0;
-}
 
 // Measured on MI355X at the 7B shapes: one row (one gate/up pair) per wave, two passes in flight, 8 waves sharing the
 // staged activations; long rows (K > 8192) want 16 waves for the staging and a third pass in flight.
@@ -351,7 +363,6 @@ GemvPlan plan_for(int K, int rows) {
     plan.waves = K > 8192 ? 16 : 8;
     plan.rows = rows;
     plan.depth = K > 8192 ? 3 : 2;
-    plan.groups = 1;
     return plan;
 }
 
@@ -360,11 +371,9 @@ int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan
     static const int forced_w = env_int("AWQ_GEMV_WAVES");
     static const int forced_r = env_int("AWQ_GEMV_ROWS");
     static const int forced_d = env_int("AWQ_GEMV_DEPTH");
-    static const int forced_g = env_int("AWQ_GEMV_GROUPS_PER_WG");
     if (forced_w) plan.waves = forced_w;
     if (forced_r) plan.rows = forced_r;
     if (forced_d) plan.depth = forced_d;
-    if (forced_g) plan.groups = forced_g;
     if (ROPE && plan.rows < 2) plan.rows = 2;  // a rotation pair lives in one wave
 #define AWQ_CASE(W_, R_) \
     if (plan.waves == W_ && plan.rows == R_) return dispatch_depth<W_, R_, KIND, ROPE>(ctx, p, grid_y, what, plan);
