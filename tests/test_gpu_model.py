@@ -137,3 +137,28 @@ def test_schedules_can_be_mixed_within_a_sequence(pair):
     t.ctx.sync()
     got = [t.token(i) for i in range(25)]
     assert got == want
+
+
+def test_fused_gate_up_with_more_row_groups_than_workgroups(ctx):
+    """hidden_dim 4480 gives 560 row groups of 8: more than the 2 workgroups per compute unit that the norm-fused
+    gate/up kernel launches, so its workgroups walk 1 or 2 groups each (and the last group is the ragged one)."""
+    cfg = dict(dim=256, hidden_dim=4480, n_layers=1, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=48, rope_theta=10000.0)
+    img = synth.make_model_image(cfg, seed=5)
+    t = A.Transformer(ctx, image=img)
+    o = oracle.Model(img)
+    try:
+        prompt = synth.prompt_tokens(3, 4, cfg["vocab_size"])
+        t.reset(prompt)
+        o.reset(prompt)
+        for _ in range(2):
+            t.forward(gen_token=False, use_graph=False, mode=A.SCHEDULE_FUSED)
+            o.forward(gen_token=False)
+        t.ctx.sync()
+        got, want = f16(t.download("hb", cfg["hidden_dim"])), f16(o.buffer("hb", cfg["hidden_dim"]))
+        assert rel_l2(got, want) <= 1e-3
+        want_tokens, _, _ = o.generate(prompt, 24, ignore_eos=True)
+        got_tokens, _ = t.generate(prompt, 24, ignore_eos=True, use_graph=False, mode=A.SCHEDULE_FUSED)
+        assert got_tokens == want_tokens
+    finally:
+        t.close()
+        o.close()
