@@ -319,8 +319,8 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     const int groups_total = div_up(p.N, W * R);
     int gx = groups_total;
     // The norm-fused gate/up kernel stages (and normalises) x in every workgroup, and that work is what bounds it:
-    // two workgroups per compute unit walk the row groups between them (measured best at the 7B shape; the plain
-    // kernels are faster with one group per workgroup).
+    // three 4-wave workgroups per compute unit walk the row groups between them (measured best at the 7B shape; the
+    // plain kernels are faster with one group per workgroup).
     if (p.norm_w && KIND == KIND_FFN) {
         static int cus = 0;
         if (!cus) {
@@ -330,7 +330,7 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
             else
                 cus = 256;
         }
-        if (gx > 2 * cus) gx = 2 * cus;
+        if (gx > 3 * cus) gx = 3 * cus;
     }
     const dim3 grid(gx, grid_y);
     const size_t lds = (size_t)p.C * 72;  // activations + per-chunk constants
@@ -374,6 +374,7 @@ int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan
     if (forced_w) plan.waves = forced_w;
     if (forced_r) plan.rows = forced_r;
     if (forced_d) plan.depth = forced_d;
+    if (p.norm_w && KIND == KIND_FFN && !forced_w && p.K <= 8192) plan.waves = 4;  // see launch()
     if (ROPE && plan.rows < 2) plan.rows = 2;  // a rotation pair lives in one wave
 #define AWQ_CASE(W_, R_) \
     if (plan.waves == W_ && plan.rows == R_) return dispatch_depth<W_, R_, KIND, ROPE>(ctx, p, grid_y, what, plan);

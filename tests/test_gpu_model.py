@@ -140,8 +140,8 @@ def test_schedules_can_be_mixed_within_a_sequence(pair):
 
 
 def test_fused_gate_up_with_more_row_groups_than_workgroups(ctx):
-    """hidden_dim 4480 gives 560 row groups of 8: more than the 2 workgroups per compute unit that the norm-fused
-    gate/up kernel launches, so its workgroups walk 1 or 2 groups each (and the last group is the ragged one)."""
+    """hidden_dim 4480 gives 1120 row groups of 4: more than the 3 workgroups per compute unit that the norm-fused
+    gate/up kernel launches, so its workgroups walk 1 or 2 groups each on a 256-CU part (and the last group is the ragged one)."""
     cfg = dict(dim=256, hidden_dim=4480, n_layers=1, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=48, rope_theta=10000.0)
     img = synth.make_model_image(cfg, seed=5)
     t = A.Transformer(ctx, image=img)
