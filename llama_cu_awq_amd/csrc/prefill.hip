@@ -54,15 +54,17 @@ __device__ __forceinline__ u32x4 permute8(const u32x4 v) {
 }
 
 // 8 nibbles of one dword -> 8 dequantised fp16 weights in the order (w0,w4)(w1,w5)(w2,w6)(w3,w7).
-__device__ __forceinline__ u32x4 dequant8(uint32_t d, uint32_t z, h16x2 s2) {
+// magic = 0x64006400 held in a vector register: v_and_or_b32 takes no literal, and with the constant in a register
+// the mask-and-merge of a nibble pair is one instruction.
+__device__ __forceinline__ u32x4 dequant8(uint32_t d, uint32_t z, h16x2 s2, uint32_t magic) {
     const h16x2 zlo = as_h2(0xE400E400u | (z * 0x00010001u));  // -(1024 + z)
     const h16x2 zhi = as_h2(0xD400D400u | (z * 0x00100010u));  // -(64 + z)
     const h16x2 sixteenth = {(h16_t)0.0625f, (h16_t)0.0625f};
     const uint32_t d8 = d >> 8;
-    const h16x2 t0 = as_h2((d & 0x000F000Fu) | 0x64006400u) + zlo;                                      // exact q - z
-    const h16x2 t1 = __builtin_elementwise_fma(as_h2((d & 0x00F000F0u) | 0x64006400u), sixteenth, zhi);  // exact
-    const h16x2 t2 = as_h2((d8 & 0x000F000Fu) | 0x64006400u) + zlo;
-    const h16x2 t3 = __builtin_elementwise_fma(as_h2((d8 & 0x00F000F0u) | 0x64006400u), sixteenth, zhi);
+    const h16x2 t0 = as_h2((d & 0x000F000Fu) | magic) + zlo;                                      // exact q - z
+    const h16x2 t1 = __builtin_elementwise_fma(as_h2((d & 0x00F000F0u) | magic), sixteenth, zhi);  // exact
+    const h16x2 t2 = as_h2((d8 & 0x000F000Fu) | magic) + zlo;
+    const h16x2 t3 = __builtin_elementwise_fma(as_h2((d8 & 0x00F000F0u) | magic), sixteenth, zhi);
     return u32x4{as_u32(t0 * s2), as_u32(t1 * s2), as_u32(t2 * s2), as_u32(t3 * s2)};  // one rounding each
 }
 
@@ -183,6 +185,8 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
     const size_t s_row = (size_t)(wb.row0 + lrow) * p.sh;  // index of the row's first scale (scales travel as aligned dwords)
     const int n_groups = p.sh;
 
+    uint32_t magic = 0x64006400u;
+    asm("" : "+v"(magic));
     f32x16 acc[4];
 #pragma unroll
     for (int i = 0; i < 4; i++)
@@ -227,7 +231,7 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
         const h16x2 s2 = {sh, sh};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const h16x8 bf = __builtin_bit_cast(h16x8, unpermute8(dequant8(wq[j], z, s2)));
+            const h16x8 bf = __builtin_bit_cast(h16x8, unpermute8(dequant8(wq[j], z, s2, magic)));
             const int chunk = j + 4 * lhalf;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
