@@ -38,6 +38,10 @@ struct GemmParams {
     int ksplit;                  // 1, or 2: two workgroups share a tile, each taking half of K
     float* part;                 // ksplit == 2: fp32 partial tiles [tile][2][128 x 128]
     unsigned int* part_counter;  // ksplit == 2: arrivals per tile, zero between launches
+    // QKV with 128-wide heads: RoPE of the q and k tiles (one head each) in the epilogue, (cos, sin) from the table
+    // [position][pair]; row m of the GEMM is position rope_pos0 + m.  Null: no rotation.
+    const float2* rope;
+    int rope_pos0;
     uint16_t* out[3];
     long long ldo[3];       // output row stride in elements
     long long out_off[3];   // element offset of output row 0 (KV cache: loff + pos0 * kv_dim)
@@ -324,6 +328,38 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
         return;
     }
     const int mat = wb.mat;
+    if (p.rope && mat < 2) {
+        // The tile is one head: column c < 64 rotates with column c + 64, which the wave two further on holds in the
+        // same lane and accumulator element.  Values are rounded to fp16 first and rotated in fp32, as the separate
+        // kernel does on the stored q and k (gpu_kernels.h:351-361); the exchange goes through the idle LDS rings.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        float* xch = reinterpret_cast<float*>(lds_bytes);  // [4 waves][64 values][64 lanes]
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                acc[i][j] = half_bits_to_float(float_to_half_bits(acc[i][j]));
+                xch[(wave * 64 + i * 16 + j) * 64 + lane] = acc[i][j];
+            }
+        __syncthreads();
+        uint16_t* ro = (mat == 0 ? p.out[0] : p.out[1]) + (size_t)(mat == 0 ? p.out_off[0] : p.out_off[1]) + wb.row0 + col;
+        const size_t rld = (size_t)(mat == 0 ? p.ldo[0] : p.ldo[1]);
+        const int pair = (wave & 1) * 32 + col;  // 0 .. 63
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                const int m = m0 + i * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+                if (m >= p.M) continue;
+                const float2 cs = p.rope[(size_t)(p.rope_pos0 + m) * 64 + pair];
+                const float other = xch[((wave ^ 2) * 64 + i * 16 + j) * 64 + lane];
+                const float v = wave < 2 ? acc[i][j] * cs.x - other * cs.y : other * cs.y + acc[i][j] * cs.x;
+                ro[(size_t)m * rld] = float_to_half_bits(v);
+            }
+        }
+        return;
+    }
     uint16_t* o = (mat == 0 ? p.out[0] : (mat == 1 ? p.out[1] : p.out[2])) +
                   (size_t)(mat == 0 ? p.out_off[0] : (mat == 1 ? p.out_off[1] : p.out_off[2])) + wb.row0 + col;
     const size_t ld = (size_t)(mat == 0 ? p.ldo[0] : (mat == 1 ? p.ldo[1] : p.ldo[2]));
@@ -748,9 +784,11 @@ int awq_launch_gemm_single(awq_ctx* ctx, uint16_t* out, long long ldo, const uin
 
 int awq_launch_gemm_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, long long kv_row0_off,
                         const uint16_t* A, int lda, int M, const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw,
-                        int K, int Nq, int Nkv) {
+                        int K, int Nq, int Nkv, const float2* rope128, int pos0) {
     pf::GemmParams p;
     gemm_common(p, A, lda, M, K, pf::EPI_QKV);
+    p.rope = rope128;  // non-null only with 128-wide heads
+    p.rope_pos0 = pos0;
     set_mat(p, 0, qw, Nq, q, Nq, 0);
     set_mat(p, 1, kw, Nkv, key_cache, Nkv, kv_row0_off);
     set_mat(p, 2, vw, Nkv, value_cache, Nkv, kv_row0_off);

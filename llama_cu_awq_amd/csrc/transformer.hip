@@ -33,7 +33,7 @@ int awq_launch_gemm_single(awq_ctx* ctx, uint16_t* out, long long ldo, const uin
                            int K, int N, int accum);
 int awq_launch_gemm_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, long long kv_row0_off,
                         const uint16_t* A, int lda, int M, const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw,
-                        int K, int Nq, int Nkv);
+                        int K, int Nq, int Nkv, const float2* rope128, int pos0);
 int awq_launch_gemm_ffn(awq_ctx* ctx, uint16_t* hb, const uint16_t* A, int lda, int M, const awq_qweight* gate_w,
                         const awq_qweight* up_w, int K, int N);
 int awq_launch_embed_rows(awq_ctx* ctx, uint16_t* x, const uint16_t* table, int dim, const int* tokens, int pos0, int M);
@@ -733,11 +733,13 @@ int awq_transformer_prefill(awq_transformer* t, int n_tokens, int gen_token) {
             const awq_layer_weights& L = t->layers[l];
             const long long loff = (long long)l * p.seq_len * kv_dim;
             if ((r = awq_launch_rmsnorm_rows(ctx, t->pf_xb, t->pf_x, L.rms_att_weight, dim, M))) return r;
+            // 128-wide heads: the QKV GEMM rotates q and k in its epilogue; other head sizes run the RoPE kernel
+            const float2* rope128 = (hs == 128) ? t->rope_table : nullptr;
             if ((r = awq_launch_gemm_qkv(ctx, t->pf_q, t->s.key_cache, t->s.value_cache, loff + (long long)pos0 * kv_dim, t->pf_xb,
-                                         dim, M, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, kv_dim)))
+                                         dim, M, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, kv_dim, rope128, pos0)))
                 return r;
-            if ((r = awq_launch_rope_rows(ctx, t->pf_q, t->s.key_cache + loff, p.n_heads, p.n_kv_heads, hs, pos0, p.rope_theta, M,
-                                          t->rope_table)))
+            if (!rope128 && (r = awq_launch_rope_rows(ctx, t->pf_q, t->s.key_cache + loff, p.n_heads, p.n_kv_heads, hs, pos0,
+                                                      p.rope_theta, M, t->rope_table)))
                 return r;
             if ((r = awq_launch_attn_prefill(ctx, t->pf_att, t->pf_q, t->s.key_cache + loff, t->s.value_cache + loff, p.n_heads, hs,
                                              kv_mul, M, pos0)))
