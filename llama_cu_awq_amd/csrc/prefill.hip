@@ -615,36 +615,73 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, c
 #pragma unroll
         for (int f = 0; f < 8; f++) qf[f] = *reinterpret_cast<const h16x8*>(qrow + f * 16);
     }
-    for (int kb = wave; kb * 32 < nk_pad; kb += 4) {
-        const uint16_t* krow = kh + (size_t)min(kb * 32 + l32, nk - 1) * kv_dim + lh * 8;
-        h16x8 kf[8];
+    {
+        // each wave takes key blocks wave, wave + 4, ...; the next block's rows are requested before this one is multiplied
+        auto load_k = [&](h16x8 (&kf)[8], int kb) {
+            const uint16_t* krow = kh + (size_t)min(kb * 32 + l32, nk - 1) * kv_dim + lh * 8;
 #pragma unroll
-        for (int f = 0; f < 8; f++) kf[f] = *reinterpret_cast<const h16x8*>(krow + f * 16);
-        f32x16 acc;
+            for (int f = 0; f < 8; f++) kf[f] = *reinterpret_cast<const h16x8*>(krow + f * 16);
+        };
+        h16x8 kf[8], kn[8];
+        if (wave * 32 < nk_pad) load_k(kf, wave);
+        for (int kb = wave; kb * 32 < nk_pad; kb += 4) {
+            const bool more = (kb + 4) * 32 < nk_pad;
+            if (more) load_k(kn, kb + 4);
+            f32x16 acc;
 #pragma unroll
-        for (int j = 0; j < 16; j++) acc[j] = 0.0f;
+            for (int j = 0; j < 16; j++) acc[j] = 0.0f;
 #pragma unroll
-        for (int f = 0; f < 8; f++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[f], kf[f], acc, 0, 0, 0);
+            for (int f = 0; f < 8; f++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[f], kf[f], acc, 0, 0, 0);
 #pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const int row = (j >> 2) * 8 + lh * 4 + (j & 3);
-            S[row * s_stride + kb * 32 + l32] = float_to_half_bits(acc[j] * alpha);
+            for (int j = 0; j < 16; j++) {
+                const int row = (j >> 2) * 8 + lh * 4 + (j & 3);
+                S[row * s_stride + kb * 32 + l32] = float_to_half_bits(acc[j] * alpha);
+            }
+            if (more) {
+#pragma unroll
+                for (int f = 0; f < 8; f++) kf[f] = kn[f];
+            }
         }
     }
     __syncthreads();
     // 2. softmax per query row (wave w takes rows w, w+4, ...); rows past nq get all-zero probabilities
     for (int qi = wave; qi < AQ; qi += 4) {
         const int size = qi < nq ? pos0 + mq0 + qi + 1 : 0;
+        uint16_t* srow = S + qi * s_stride;
         float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed
-        for (int t = lane; t < size; t += 64) m = fmaxf(m, half_bits_to_float(S[qi * s_stride + t]));
+        if (nk_pad <= 512) {
+            // up to 8 scores per lane stay in registers: one exponential per score instead of two
+            float v[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const int t = lane + 64 * k;
+                v[k] = t < size ? half_bits_to_float(srow[t]) : -INFINITY;
+                m = fmaxf(m, v[k]);
+            }
+            m = wave_max(m);
+            float sum = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                v[k] = lane + 64 * k < size ? expf(v[k] - m) : 0.0f;
+                sum += v[k];
+            }
+            sum = wave_sum(sum);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const int t = lane + 64 * k;
+                if (t < nk_pad) srow[t] = float_to_half_bits(t < size ? v[k] / sum : 0.0f);
+            }
+            continue;
+        }
+        for (int t = lane; t < size; t += 64) m = fmaxf(m, half_bits_to_float(srow[t]));
         m = wave_max(m);
         float sum = 0.0f;
-        for (int t = lane; t < size; t += 64) sum += expf(half_bits_to_float(S[qi * s_stride + t]) - m);
+        for (int t = lane; t < size; t += 64) sum += expf(half_bits_to_float(srow[t]) - m);
         sum = wave_sum(sum);
         for (int t = lane; t < nk_pad; t += 64) {
             float pv = 0.0f;
-            if (t < size) pv = expf(half_bits_to_float(S[qi * s_stride + t]) - m) / sum;
-            S[qi * s_stride + t] = float_to_half_bits(pv);
+            if (t < size) pv = expf(half_bits_to_float(srow[t]) - m) / sum;
+            srow[t] = float_to_half_bits(pv);
         }
     }
     // 3. O = P V.  Loader role (threads 0..127): 8 keys x 8 dims, transposed in registers.
