@@ -687,15 +687,16 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, c
     // 3. O = P V.  Loader role (threads 0..127): 8 keys x 8 dims, transposed in registers.
     const int kg = tid & 7, dc = (tid >> 3) & 15;
     const bool loader = tid < 128;
-    u32x4 vr[8];
-    auto load_v = [&](int t0) {
+    // value rows travel two blocks of 64 keys ahead of the multiply, in two register sets
+    u32x4 va[8], vb[8];
+    auto load_v = [&](u32x4 (&vr)[8], int t0) {
         if (loader) {
 #pragma unroll
             for (int r = 0; r < 8; r++)
                 vr[r] = *reinterpret_cast<const u32x4*>(vh + (size_t)min(t0 + kg * 8 + r, nk - 1) * kv_dim + dc * 8);
         }
     };
-    auto store_v = [&](int buf) {
+    auto store_v = [&](const u32x4 (&vr)[8], int buf) {
         if (loader) {
             uint16_t* vt = Vt + buf * (HS * VT_STRIDE);
 #pragma unroll
@@ -711,12 +712,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, c
     f32x16 oacc;
 #pragma unroll
     for (int j = 0; j < 16; j++) oacc[j] = 0.0f;
-    load_v(0);
-    store_v(0);
-    __syncthreads();  // also orders the probabilities written above
-    for (int t0 = 0, buf = 0; t0 < nk_pad; t0 += 64, buf ^= 1) {
-        const bool more = t0 + 64 < nk_pad;
-        if (more) load_v(t0 + 64);
+    auto multiply = [&](int t0, int buf) {
         const uint16_t* vt = Vt + buf * (HS * VT_STRIDE);
 #pragma unroll
         for (int kc = 0; kc < 4; kc++) {
@@ -724,7 +720,22 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, c
             const h16x8 vf = *reinterpret_cast<const h16x8*>(&vt[(wave * 32 + l32) * VT_STRIDE + kc * 16 + lh * 8]);
             oacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(pf, vf, oacc, 0, 0, 0);
         }
-        if (more) store_v(buf ^ 1);
+    };
+    load_v(va, 0);
+    if (64 < nk_pad) load_v(vb, 64);
+    store_v(va, 0);
+    if (128 < nk_pad) load_v(va, 128);
+    __syncthreads();  // also orders the probabilities written above
+    // blocks alternate between the register sets: block k (keys 64k ..) is in set k & 1 and LDS buffer k & 1
+    for (int t0 = 0; t0 < nk_pad; t0 += 128) {
+        multiply(t0, 0);
+        if (t0 + 64 < nk_pad) store_v(vb, 1);
+        if (t0 + 192 < nk_pad) load_v(vb, t0 + 192);
+        __syncthreads();
+        if (t0 + 64 >= nk_pad) break;
+        multiply(t0 + 64, 1);
+        if (t0 + 128 < nk_pad) store_v(va, 0);
+        if (t0 + 256 < nk_pad) load_v(va, t0 + 256);
         __syncthreads();
     }
 #pragma unroll
