@@ -12,10 +12,6 @@ struct awq_ctx {
     int device;
     hipStream_t stream;
     bool owns_stream;
-    // Library workspace for the split attention kernel: per-(head, split)
-    // partial outputs and one arrival counter per head (self-resetting).
-    float* attn_partial;
-    unsigned int* attn_counter;
     // Workspace of the prefill GEMM's split-K form (allocated on first use): fp32 partial tiles and per-tile arrival
     // counters (self-resetting).
     float* gemm_part;
@@ -25,9 +21,7 @@ struct awq_ctx {
 };
 
 constexpr int kAttnMaxHeads = 256;
-constexpr int kAttnMaxSplits = 16;
-constexpr int kAttnMaxHeadSize = 256;
-constexpr int kAttnFusedMaxSeq = 512;  // up to this launch size attention runs as one workgroup per head
+constexpr int kAttnFusedMaxSeq = 256;  // up to this launch size attention runs as one workgroup per head
 
 void awq_set_error(const char* fmt, ...);
 

@@ -115,100 +115,87 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(uint16_t* att, const u
     }
 }
 
-// Pass 2: softmax statistics (recomputed by every workgroup of a head from the fp16 scores: a few KB),
-// probabilities rounded to fp16 as the reference does, and P.V over this workgroup's slice of positions.  The slice
-// is sized so that its value rows are requested in one go, before the statistics are computed.  With more than one
-// split the per-split partial sums are written through to memory and combined, in split order, by the last workgroup
-// of the head to arrive.
-template <int LP>
-__global__ __launch_bounds__(256) void attn_softmax_pv_kernel(uint16_t* output, const uint16_t* att,
-                                                              const uint16_t* value_cache, int head_size, int kv_mul,
-                                                              int row_stride, const int* pPos, float* partial,
-                                                              unsigned int* counter) {
-    __shared__ float red[4];
-    __shared__ float acc_lds[4][kAttnMaxHeadSize];
-    __shared__ unsigned int arrival;
+// Pass 2: softmax and P.V.  A workgroup of 16 waves owns LR * 8 of a head's dimensions (LR lanes x 16 bytes of every
+// value row) over ALL positions, so no partial sums leave the workgroup.  The 1024 / LR lane groups take positions
+// g, g + 1024 / LR, ...; a lane requests R rows at once, after the scores of those positions (loads return in order
+// and the softmax statistics need only the scores; each position is counted by one lane of its group).
+template <int LR, int R>
+__global__ __launch_bounds__(1024) void attn_pv_sliced_kernel(uint16_t* output, const uint16_t* att, const uint16_t* value_cache,
+                                                              int num_heads, int head_size, int kv_mul, int row_stride,
+                                                              const int* pPos) {
+    constexpr int NG = 1024 / LR;  // lane groups = positions per pass
+    constexpr int SW = LR * 8;     // dimensions per workgroup
+    __shared__ float red[16];
+    __shared__ float acc_lds[16][SW];
     const int size = *pPos + 1;
-    const int h = blockIdx.y;
-    const int nsplit = gridDim.x;
-    const int split = blockIdx.x;
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
+    // heads along x (the grid is padded to a multiple of 8 of them): the slices of a head share an XCD and its L2
+    const int h = blockIdx.x, slice = blockIdx.y;
+    if (h >= num_heads) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int pg = tid / LR, ql = tid % LR;
     const uint16_t* a = att + (size_t)h * size;
-
-    // the head's scores: 8 per thread requested together cover 2048 positions, a loop takes the rest.  They are
-    // requested ahead of the value rows because loads return in order and the statistics need only the scores.
-    constexpr int SP = 8;
-    uint16_t sv[SP];
+    const uint16_t* vh = value_cache + (size_t)(h / kv_mul) * head_size + slice * SW + ql * 8;
+    u32x4 vv[R];
+    uint16_t sv[R];
+    auto request = [&](int t0) {
 #pragma unroll
-    for (int i = 0; i < SP; i++) {
-        const int t = i * 256 + tid;
-        sv[i] = a[min(t, size - 1)];
-    }
-    // this workgroup's positions; a round covers 64 of them (4 waves x PW positions x 4 loads per lane)
-    const int per = (size + nsplit - 1) / nsplit;
-    const int tb = split * per;
-    const int te = min(size, tb + per);
-    constexpr int PW = 64 / LP;
-    const int j = lane % LP;
-    const int pr = lane / LP;
-    const uint16_t* vh = value_cache + (size_t)(h / kv_mul) * head_size + j * 8;
-    const int tfirst = tb + wave * PW + pr;
-    u32x4 vfirst[4];
-    uint16_t afirst[4];
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const int t = tfirst + k * 4 * PW;
-        if (t < te) {
-            vfirst[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
-            afirst[k] = a[t];
+        for (int k = 0; k < R; k++) {
+            const int t = t0 + pg + NG * k;
+            if (t < size) sv[k] = a[t];
         }
-    }
-
-    // max (the reference seeds idle threads of its 1024-thread block with 0)
-    float m = (size < 1024) ? 0.0f : -INFINITY;
 #pragma unroll
-    for (int i = 0; i < SP; i++)
-        if (i * 256 + tid < size) m = fmaxf(m, half_bits_to_float(sv[i]));
-    for (int t = SP * 256 + tid; t < size; t += 256) m = fmaxf(m, half_bits_to_float(a[t]));
+        for (int k = 0; k < R; k++) {
+            const int t = t0 + pg + NG * k;
+            if (t < size) vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+        }
+    };
+    request(0);
+    // statistics over all positions (gpu_kernels.h:376-400; the max seed is the reference's idle-lane 0 when its
+    // 1024-thread block is not full)
+    float m = (size < 1024) ? 0.0f : -INFINITY;
+    if (ql == 0) {
+#pragma unroll
+        for (int k = 0; k < R; k++)
+            if (pg + NG * k < size) m = fmaxf(m, half_bits_to_float(sv[k]));
+        for (int t = pg + NG * R; t < size; t += NG) m = fmaxf(m, half_bits_to_float(a[t]));
+    }
     m = wave_max(m);
     if (lane == 0) red[wave] = m;
     __syncthreads();
-    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+#pragma unroll
+    for (int w = 0; w < 16; w++) m = fmaxf(m, red[w]);
     __syncthreads();
     float sum = 0.0f;
+    if (ql == 0) {
 #pragma unroll
-    for (int i = 0; i < SP; i++)
-        if (i * 256 + tid < size) sum += expf(half_bits_to_float(sv[i]) - m);
-    for (int t = SP * 256 + tid; t < size; t += 256) sum += expf(half_bits_to_float(a[t]) - m);
+        for (int k = 0; k < R; k++)
+            if (pg + NG * k < size) sum += expf(half_bits_to_float(sv[k]) - m);
+        for (int t = pg + NG * R; t < size; t += NG) sum += expf(half_bits_to_float(a[t]) - m);
+    }
     sum = wave_sum(sum);
     if (lane == 0) red[wave] = sum;
     __syncthreads();
-    sum = (red[0] + red[1]) + (red[2] + red[3]);
+    {
+        float r[16];
+#pragma unroll
+        for (int w = 0; w < 16; w++) r[w] = red[w];
+#pragma unroll
+        for (int n = 16; n > 1; n >>= 1)
+#pragma unroll
+            for (int i = 0; i < n / 2; i++) r[i] = r[2 * i] + r[2 * i + 1];
+        sum = r[0];
+    }
 
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.0f;
-    for (int t0 = tfirst; t0 - pr - wave * PW < te; t0 += 16 * PW) {
-        u32x4 vv[4];
-        uint16_t av[4];
+    for (int t0 = 0; t0 < size; t0 += NG * R) {
+        if (t0) request(t0);
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int t = t0 + k * 4 * PW;
-            if (t0 == tfirst) {
-                vv[k] = vfirst[k];
-                av[k] = afirst[k];
-            } else if (t < te) {
-                vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
-                av[k] = a[t];
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int t = t0 + k * 4 * PW;
-            if (t < te) {
-                const float e = expf(half_bits_to_float(av[k]) - m);
+        for (int k = 0; k < R; k++) {
+            const int t = t0 + pg + NG * k;
+            if (t < size) {
+                const float e = expf(half_bits_to_float(sv[k]) - m);
                 const float p = half_bits_to_float(float_to_half_bits(e / sum));  // probability rounded to fp16
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -219,46 +206,30 @@ __global__ __launch_bounds__(256) void attn_softmax_pv_kernel(uint16_t* output, 
             }
         }
     }
-    // combine the PW position groups of the wave, then the 4 waves
+    // add up the lane groups of the wave (lanes with the same lane % LR), then the 16 waves
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        for (int off = LP; off < 64; off <<= 1) acc[i] += __shfl_xor(acc[i], off);
+        if (LR <= 1) acc[i] += dpp_mov<0xB1>(acc[i]);   // quad_perm [1,0,3,2]
+        if (LR <= 2) acc[i] += dpp_mov<0x4E>(acc[i]);   // quad_perm [2,3,0,1]
+        if (LR <= 4) acc[i] += dpp_mov<0x124>(acc[i]);  // row_ror:4
+        if (LR <= 8) acc[i] += dpp_mov<0x128>(acc[i]);  // row_ror:8
+        acc[i] += __shfl_xor(acc[i], 16);
+        acc[i] += __shfl_xor(acc[i], 32);
     }
-    if (pr == 0) {
+    if (lane < LR) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) acc_lds[wave][j * 8 + i] = acc[i];
+        for (int i = 0; i < 8; i++) acc_lds[wave][lane * 8 + i] = acc[i];
     }
     __syncthreads();
-    float total = 0.0f;
-    if (tid < head_size) total = (acc_lds[0][tid] + acc_lds[1][tid]) + (acc_lds[2][tid] + acc_lds[3][tid]);
-
-    if (nsplit == 1) {
-        if (tid < head_size) output[(size_t)h * head_size + tid] = float_to_half_bits(total);
-        return;
-    }
-    // Publish this split's partial sums: written through at agent scope (a release fence per workgroup would flush
-    // the whole L2 each time), waited for, then counted in.
-    float* my = partial + ((size_t)h * kAttnMaxSplits + split) * kAttnMaxHeadSize;
-    if (tid < head_size) __hip_atomic_store(&my[tid], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (tid == 0) arrival = __hip_atomic_fetch_add(&counter[h], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (arrival == (unsigned int)(nsplit - 1)) {
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        if (tid < head_size) {
-            const float* ph = partial + (size_t)h * kAttnMaxSplits * kAttnMaxHeadSize;
-            // all partials are requested before the first is used (each is a trip to memory)
-            float pv[kAttnMaxSplits];
+    if (tid < SW) {
+        float r[16];
 #pragma unroll
-            for (int sp = 0; sp < kAttnMaxSplits; sp++) pv[sp] = sp < nsplit ? ph[(size_t)sp * kAttnMaxHeadSize + tid] : 0.0f;
-            float s = 0.0f;
+        for (int w = 0; w < 16; w++) r[w] = acc_lds[w][tid];
 #pragma unroll
-            for (int sp = 0; sp < kAttnMaxSplits; sp++)
-                if (sp < nsplit) s += pv[sp];
-            output[(size_t)h * head_size + tid] = float_to_half_bits(s);
-        }
-        if (tid == 0) counter[h] = 0;  // ready for the next launch
+        for (int n = 16; n > 1; n >>= 1)
+#pragma unroll
+            for (int i = 0; i < n / 2; i++) r[i] = r[2 * i] + r[2 * i + 1];
+        output[(size_t)h * head_size + slice * SW + tid] = float_to_half_bits(r[0]);
     }
 }
 
@@ -469,14 +440,12 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
     hipLaunchKernelGGL((attn_scores_kernel<LP>), dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, ctx->stream, att, q,
                        key_cache, head_size, kv_mul, row_stride, alpha, pos);
     if (int r = awq_check_launch("attn_scores")) return r;
-    // one or two rounds of value rows per workgroup; more than 16 splits cost more in the exchange of partial sums
-    // (same-address arrivals, partials to add) than the extra workgroups bring
-    int nsplit = div_up(max_seq_len, 128);
-    if (nsplit > kAttnMaxSplits) nsplit = kAttnMaxSplits;
-    if (nsplit < 1) nsplit = 1;
-    hipLaunchKernelGGL((attn_softmax_pv_kernel<LP>), dim3(nsplit, num_heads), dim3(256), 0, ctx->stream, output, att,
-                       value_cache, head_size, kv_mul, row_stride, pos, ctx->attn_partial, ctx->attn_counter);
-    return awq_check_launch("attn_softmax_pv");
+    // 16 dimensions (2 lanes x 16 bytes of a row) per workgroup measured best (32: -2.5 %, 8: -4 %, 64: -12 % tokens/s
+    // at the 13B shape, 1.6 K context); the head count is padded to a multiple of 8 so that the slices of a head
+    // (ids h, h + padded heads, ...) share an XCD and the cache lines they split between them
+    hipLaunchKernelGGL((attn_pv_sliced_kernel<2, 4>), dim3((num_heads + 7) & ~7, LP / 2), dim3(1024), 0, ctx->stream, output, att,
+                       value_cache, num_heads, head_size, kv_mul, row_stride, pos);
+    return awq_check_launch("attn_pv_sliced");
 }
 
 }  // namespace

@@ -56,24 +56,10 @@ static int ctx_init(int device, hipStream_t stream, bool owns, awq_ctx** out) {
     c->device = device;
     c->stream = stream;
     c->owns_stream = owns;
-    c->attn_partial = nullptr;
-    c->attn_counter = nullptr;
     c->gemm_part = nullptr;
     c->gemm_part_bytes = 0;
     c->gemm_counter = nullptr;
     c->gemm_counter_count = 0;
-    size_t partial_bytes = (size_t)kAttnMaxHeads * kAttnMaxSplits * kAttnMaxHeadSize * sizeof(float);
-    hipError_t e = hipMalloc((void**)&c->attn_partial, partial_bytes);
-    if (e == hipSuccess) e = hipMalloc((void**)&c->attn_counter, kAttnMaxHeads * sizeof(unsigned int));
-    if (e == hipSuccess) e = hipMemset(c->attn_counter, 0, kAttnMaxHeads * sizeof(unsigned int));
-    if (e != hipSuccess) {
-        awq_set_error("context workspace allocation failed: %s", hipGetErrorString(e));
-        if (c->attn_partial) (void)hipFree(c->attn_partial);
-        if (c->attn_counter) (void)hipFree(c->attn_counter);
-        if (owns) (void)hipStreamDestroy(stream);
-        delete c;
-        return AWQ_ERR_HIP;
-    }
     *out = c;
     return AWQ_OK;
 }
@@ -98,8 +84,6 @@ int awq_ctx_create_on_stream(int device, void* hip_stream, awq_ctx** out) {
 int awq_ctx_destroy(awq_ctx* ctx) {
     if (int r = awq_bind(ctx)) return r;
     (void)hipStreamSynchronize(ctx->stream);
-    (void)hipFree(ctx->attn_partial);
-    (void)hipFree(ctx->attn_counter);
     if (ctx->gemm_part) (void)hipFree(ctx->gemm_part);
     if (ctx->gemm_counter) (void)hipFree(ctx->gemm_counter);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
