@@ -119,6 +119,10 @@ constexpr int GEMM_LDS_BYTES = A_STAGES * TILE_BYTES + W_STAGES * W_STAGE_BYTES;
 __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_byte_off) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_byte_off), "v"(gptr) : "memory");
 }
+// Same with the address as a wave-uniform base plus a 32-bit byte offset per lane (no 64-bit vector arithmetic).
+__device__ __forceinline__ void dma16(const void* sbase, uint32_t voff, uint32_t lds_byte_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_off), "v"(voff), "s"(sbase) : "memory");
+}
 __device__ __forceinline__ void dma4(const void* gptr, uint32_t lds_byte_off) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_byte_off), "v"(gptr) : "memory");
 }
@@ -162,12 +166,12 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
 
     // activation loader: wave w, instruction q covers tile rows (4w + q) * 8 .. + 8 (8 lanes x 16 bytes per row);
     // the lane's LDS chunk is lane & 7, so it fetches the source chunk that the swizzle maps there
-    const uint16_t* a_src[4];
+    uint32_t a_off[4];  // byte offsets from p.A (a chunk of activations is far below 4 GB)
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         const int r = (wave * 4 + q) * 8 + (lane >> 3);
         const int c = (lane & 7) ^ lds_key(r);
-        a_src[q] = p.A + (size_t)min(m0 + r, p.M - 1) * p.lda + c * 8;  // rows past M are computed, never stored
+        a_off[q] = (uint32_t)(((size_t)min(m0 + r, p.M - 1) * p.lda + c * 8) * 2);  // rows past M are computed, never stored
     }
     // weight loader: instruction q of a pair of steps covers the wave's rows 16q .. 16q+15, 4 lanes x 16 bytes per
     // row; 16-byte unit u of a row's 64 bytes sits at LDS unit u ^ ((row >> 1) & 3) (bank spread for the reads below)
@@ -207,7 +211,7 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
         const int k0 = min(step * BK, k_last);
         const uint32_t dst = (uint32_t)((step % A_STAGES) * TILE_BYTES + wave * 4096);
 #pragma unroll
-        for (int q = 0; q < 4; q++) dma16(a_src[q] + k0, dst + q * 1024);
+        for (int q = 0; q < 4; q++) dma16(p.A + k0, a_off[q], dst + q * 1024);
     };
     auto load_w = [&](int pair) {  // 4 loads: K range [128 * pair, 128 * pair + 128) of the wave's 32 rows
         const uint32_t dst = W_RING + (uint32_t)((pair % W_STAGES) * W_STAGE_BYTES + wave * W_WAVE_BYTES);
@@ -768,6 +772,10 @@ static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* 
             return AWQ_ERR_HIP;
         }
         lds_raised = true;
+    }
+    if ((size_t)p.M * (size_t)p.lda * 2 >= ((size_t)1 << 32)) {  // the kernel addresses A by 32-bit byte offsets
+        awq_set_error("%s: activation block of %d x %d halves exceeds 4 GB", what, p.M, p.lda);
+        return AWQ_ERR_SHAPE;
     }
     p.mtiles = div_up(p.M, pf::BM);
     p.ntiles = ntiles;
