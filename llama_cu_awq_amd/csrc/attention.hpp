@@ -102,8 +102,11 @@ __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att
         }
     }
 #pragma unroll
-    for (int i = 0; i < 8; i++)
-        for (int off = LP; off < 64; off <<= 1) acc[i] += __shfl_xor(acc[i], off);
+    for (int i = 0; i < 8; i++) {
+        if (LP <= 8) acc[i] = lane_xor_sum<8>(acc[i]);
+        if (LP <= 16) acc[i] = lane_xor_sum<16>(acc[i]);
+        acc[i] = lane_xor_sum<32>(acc[i]);
+    }
     if (pr == 0) {
 #pragma unroll
         for (int i = 0; i < 8; i++) acc_lds[wave * head_size + j * 8 + i] = acc[i];

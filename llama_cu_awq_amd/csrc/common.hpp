@@ -101,6 +101,28 @@ __device__ __forceinline__ float read_lane(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
+// The row and half swaps of gfx950: v_permlane16_swap exchanges the odd rows (of 16 lanes) of its first operand with
+// the even rows of the second, v_permlane32_swap the upper half of the first with the lower half of the second.  Fed
+// the same value twice (in two registers) they leave the lane's own value in one and its partner's (lane ^ 16, lane ^
+// 32) in the other, in the same order in both lanes.  Inline assembly: the compiler's builtin returns its first result
+// twice; the s_nop cover the VALU-write -> permlane-read and permlane-write -> VALU-read hazards that the compiler
+// cannot see through an asm statement.
+__device__ __forceinline__ void swap16(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap32(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+// v + (v of lane ^ OFF) for OFF = 8, 16, 32 without a trip through the LDS crossbar.
+template <int OFF>
+__device__ __forceinline__ float lane_xor_sum(float v) {
+    static_assert(OFF == 8 || OFF == 16 || OFF == 32, "unsupported distance");
+    if (OFF == 8) return v + dpp_mov<0x128>(v);  // row_ror:8
+    float a = v, b = v;
+    if (OFF == 16) swap16(a, b); else swap32(a, b);
+    return a + b;
+}
+
 // Sum within each aligned group of 16 lanes (a DPP row); every lane of the
 // group ends up holding the group's sum.
 __device__ __forceinline__ float row16_sum(float v) {
@@ -115,9 +137,17 @@ __device__ __forceinline__ float wave_sum(float v) {
     v = row16_sum(v);
     return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
 }
+// Maximum over the 64 lanes, in every lane (DPP inside a row of 16, then the row and half swaps).
 __device__ __forceinline__ float wave_max(float v) {
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
+    v = fmaxf(v, dpp_mov<0xB1>(v));
+    v = fmaxf(v, dpp_mov<0x4E>(v));
+    v = fmaxf(v, dpp_mov<0x124>(v));
+    v = fmaxf(v, dpp_mov<0x128>(v));
+    float a = v, b = v;
+    swap16(a, b);
+    a = b = fmaxf(a, b);
+    swap32(a, b);
+    return fmaxf(a, b);
 }
 // Sum within aligned groups of LP lanes (LP = 8, 16 or 32).
 template <int LP>
@@ -130,7 +160,7 @@ __device__ __forceinline__ float group_sum(float v) {
     } else {
         v += dpp_mov<0x124>(v);
         v += dpp_mov<0x128>(v);
-        if (LP == 32) v += __shfl_xor(v, 16);
+        if (LP == 32) v = lane_xor_sum<16>(v);
     }
     return v;
 }

@@ -213,8 +213,8 @@ __global__ __launch_bounds__(1024) void attn_pv_sliced_kernel(uint16_t* output, 
         if (LR <= 2) acc[i] += dpp_mov<0x4E>(acc[i]);   // quad_perm [2,3,0,1]
         if (LR <= 4) acc[i] += dpp_mov<0x124>(acc[i]);  // row_ror:4
         if (LR <= 8) acc[i] += dpp_mov<0x128>(acc[i]);  // row_ror:8
-        acc[i] += __shfl_xor(acc[i], 16);
-        acc[i] += __shfl_xor(acc[i], 32);
+        acc[i] = lane_xor_sum<16>(acc[i]);
+        acc[i] = lane_xor_sum<32>(acc[i]);
     }
     if (lane < LR) {
 #pragma unroll
