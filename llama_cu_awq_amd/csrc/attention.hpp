@@ -17,10 +17,12 @@ __host__ __device__ constexpr int attention_head_lds_floats(int max_seq, int hea
 // LP = lanes per position (head_size / 8), NW = waves of the calling workgroup (all of them must call).
 // lds: attention_head_lds_floats() floats, free for use.  k_head / v_head: the head's slice of row 0 of the layer's
 // caches; rows are row_stride halves apart.
-template <int LP, int NW>
+// NS > 1: NS workgroups share a head; each computes all scores but only the P.V of the value dimensions of its slice
+// (lanes j with j / (LP / NS) == slice), so that a head's value rows come in through NS compute units.
+template <int LP, int NW, int NS = 1>
 __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att_head, const uint16_t* q_head,
                                                const uint16_t* k_head, const uint16_t* v_head, int head_size,
-                                               int row_stride, float alpha, int size, float* lds) {
+                                               int row_stride, float alpha, int size, float* lds, int slice = 0) {
     float* sc = lds;                          // [size] scores (fp16-rounded values)
     float* acc_lds = lds + ((size + 3) & ~3);  // [NW][head_size]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -31,13 +33,14 @@ __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att
     const u32x4 qv = *reinterpret_cast<const u32x4*>(q_head + j * 8);
     const uint16_t* kh = k_head + j * 8;
     const uint16_t* vh = v_head + j * 8;
+    const bool mine = NS == 1 || j / (LP / NS) == slice;  // this lane's 8 value dimensions belong to the slice
     // The value rows of the first round are requested together with its key rows: at short context that is all of
     // them, and the softmax then runs while they are on their way.
     u32x4 vfirst[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int t = tfirst + k * tstep;
-        if (t < size) vfirst[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+        if (t < size && mine) vfirst[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
     }
     for (int t0 = tfirst; t0 - tfirst < size; t0 += 4 * tstep) {
         u32x4 kv[4];
@@ -57,7 +60,7 @@ __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att
             s = group_sum<LP>(s);
             if (j == 0 && t < size) {
                 const uint16_t hb = float_to_half_bits(s * alpha);
-                att_head[t] = hb;
+                if (NS == 1 || slice == 0) att_head[t] = hb;
                 sc[t] = half_bits_to_float(hb);
             }
         }
@@ -83,13 +86,13 @@ __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att
             const int t = t0 + k * tstep;
             if (t0 == tfirst)
                 vv[k] = vfirst[k];
-            else if (t < size)
+            else if (t < size && mine)
                 vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
         }
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const int t = t0 + k * tstep;
-            if (t < size) {
+            if (t < size && mine) {
                 const float e = expf(sc[t] - m);
                 const float pv = half_bits_to_float(float_to_half_bits(e / sum));
 #pragma unroll
@@ -107,15 +110,16 @@ __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att
         if (LP <= 16) acc[i] = lane_xor_sum<16>(acc[i]);
         acc[i] = lane_xor_sum<32>(acc[i]);
     }
-    if (pr == 0) {
+    if (pr == 0 && mine) {
 #pragma unroll
         for (int i = 0; i < 8; i++) acc_lds[wave * head_size + j * 8 + i] = acc[i];
     }
     __syncthreads();
-    if (tid < head_size) {
+    const int d = NS == 1 ? tid : slice * (head_size / NS) + tid;  // output dimension of this thread
+    if (tid < head_size / NS) {
         float total = 0.0f;
 #pragma unroll
-        for (int w = 0; w < NW; w++) total += acc_lds[w * head_size + tid];
-        out_head[tid] = float_to_half_bits(total);
+        for (int w = 0; w < NW; w++) total += acc_lds[w * head_size + d];
+        out_head[d] = float_to_half_bits(total);
     }
 }

@@ -233,19 +233,23 @@ __global__ __launch_bounds__(1024) void attn_pv_sliced_kernel(uint16_t* output, 
     }
 }
 
-// Short contexts: one workgroup of 16 waves per head does scores, softmax and P.V in a single launch (the work is
-// a few hundred KB per head, so the launch count matters more than the parallelism).  Same arithmetic and
+// Short contexts: a workgroup of 16 waves does scores, softmax and P.V of a head in a single launch (the work is a few
+// hundred KB per head, so the launch count matters more than the parallelism); NS workgroups per head each take a
+// slice of the value dimensions and compute the scores redundantly.  Same arithmetic and
 // rounding points as the two-pass kernels above; the fp16 scores are also left in att.
-template <int LP>
+template <int LP, int NS>
 __global__ __launch_bounds__(1024) void attn_fused_kernel(uint16_t* output, uint16_t* att, const uint16_t* q,
-                                                          const uint16_t* key_cache, const uint16_t* value_cache, int head_size,
-                                                          int kv_mul, int row_stride, float alpha, const int* pPos) {
+                                                          const uint16_t* key_cache, const uint16_t* value_cache, int num_heads,
+                                                          int head_size, int kv_mul, int row_stride, float alpha,
+                                                          const int* pPos) {
     extern __shared__ float fsm[];
     const int size = *pPos + 1;
-    const int h = blockIdx.x;
-    attention_head<LP, 16>(output + (size_t)h * head_size, att + (size_t)h * size, q + (size_t)h * head_size,
-                           key_cache + (size_t)(h / kv_mul) * head_size, value_cache + (size_t)(h / kv_mul) * head_size,
-                           head_size, row_stride, alpha, size, fsm);
+    // heads along x, padded to a multiple of 8: the NS workgroups of a head (ids h, h + padded heads, ...) share an XCD
+    const int h = blockIdx.x, slice = blockIdx.y;
+    if (h >= num_heads) return;
+    attention_head<LP, 16, NS>(output + (size_t)h * head_size, att + (size_t)h * size, q + (size_t)h * head_size,
+                               key_cache + (size_t)(h / kv_mul) * head_size, value_cache + (size_t)(h / kv_mul) * head_size,
+                               head_size, row_stride, alpha, size, fsm, slice);
 }
 
 // ------------------------------------------------------------------ fp16 matvec
@@ -433,8 +437,9 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
     const float alpha = (float)(1.0 / sqrt((double)head_size));
     if (max_seq_len <= kAttnFusedMaxSeq) {
         const size_t lds = (size_t)attention_head_lds_floats(max_seq_len, head_size, 16) * sizeof(float);
-        hipLaunchKernelGGL((attn_fused_kernel<LP>), dim3(num_heads), dim3(1024), lds, ctx->stream, output, att, q, key_cache,
-                           value_cache, head_size, kv_mul, row_stride, alpha, pos);
+        // two workgroups per head (halves of the value dimensions): +0.4 .. 0.7 % tokens/s at 7B; four: no better
+        hipLaunchKernelGGL((attn_fused_kernel<LP, 2>), dim3((num_heads + 7) & ~7, 2), dim3(1024), lds, ctx->stream, output, att, q,
+                           key_cache, value_cache, num_heads, head_size, kv_mul, row_stride, alpha, pos);
         return awq_check_launch("attn_fused");
     }
     hipLaunchKernelGGL((attn_scores_kernel<LP>), dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, ctx->stream, att, q,
