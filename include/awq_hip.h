@@ -175,6 +175,14 @@ int awq_transformer_layer(const awq_transformer* t, int layer, awq_layer_weights
 int awq_transformer_globals(const awq_transformer* t, const uint16_t** embed, const uint16_t** wcls,
                             const uint16_t** rms_final);
 
+/* Position bookkeeping of the model-level calls.  The reference sizes each pass from the pinned position after a
+ * stream synchronisation (llama2_q4.cu:552, 713).  Here the transformer counts on the host the passes it has ISSUED
+ * (reset: 0; set_pos: pos; forward / accept / sample: +1; prefill: +n_tokens), and that count sizes the attention
+ * launch, selects the recorded sequence and bounds the position by seq_len.  Passes may therefore be issued back to
+ * back without synchronising.  A caller that advances the device position of a transformer's run state by other means
+ * (awq_argmax_advance or awq_sampler_sample on its buffers) must call awq_transformer_set_pos before the next
+ * model-level call. */
+
 /* Start a sequence (llama2_q4.cu:703-705): position 0, prompt copied into the shared token list. */
 int awq_transformer_reset(awq_transformer* t, const int* prompt_tokens, int num_prompt_tokens);
 /* Start at position `pos` with caller-provided KV-cache contents below it; `token` is consumed next. */
@@ -242,7 +250,9 @@ int awq_gemm_int4(awq_ctx* ctx, uint16_t* out, int ldo, const uint16_t* a, int l
 /* Consume the n_tokens tokens at positions pos .. pos+n_tokens-1 of the shared token list in one batched pass:
  * afterwards the KV cache rows, the logits (of the last token), the token list and the position are those that
  * n_tokens calls of awq_transformer_forward (gen_token false for all but the last, `gen_token` for the last) would
- * leave.  Needs dim, kv_dim and hidden_dim to be multiples of 128.  Synchronises the stream on entry. */
+ * leave.  Needs dim, kv_dim and hidden_dim to be multiples of 128.  The batched attention holds a score row per
+ * query in LDS and takes contexts of up to 1920 positions with 128-wide heads (5048 / 4856 with 64 / 256); prompt
+ * tokens beyond that are run one at a time through the matrix-vector path inside this call. */
 int awq_transformer_prefill(awq_transformer* t, int n_tokens, int gen_token);
 
 /* Diagnostics of the persistent schedule (no counterpart in the reference; its DUMP_PER_TOKEN_TIMINGS switch,

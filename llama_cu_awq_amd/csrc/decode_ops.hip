@@ -241,9 +241,11 @@ template <int LP, int NS>
 __global__ __launch_bounds__(1024) void attn_fused_kernel(uint16_t* output, uint16_t* att, const uint16_t* q,
                                                           const uint16_t* key_cache, const uint16_t* value_cache, int num_heads,
                                                           int head_size, int kv_mul, int row_stride, float alpha,
-                                                          const int* pPos) {
+                                                          const int* pPos, int max_seq_len) {
     extern __shared__ float fsm[];
-    const int size = *pPos + 1;
+    // LDS was sized for max_seq_len positions by the launcher; a position beyond it (a caller that sized the launch
+    // from a stale position) must not run past that
+    const int size = min(*pPos + 1, max_seq_len);
     // heads along x, padded to a multiple of 8: the NS workgroups of a head (ids h, h + padded heads, ...) share an XCD
     const int h = blockIdx.x, slice = blockIdx.y;
     if (h >= num_heads) return;
@@ -439,7 +441,7 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
         const size_t lds = (size_t)attention_head_lds_floats(max_seq_len, head_size, 16) * sizeof(float);
         // two workgroups per head (halves of the value dimensions): +0.4 .. 0.7 % tokens/s at 7B; four: no better
         hipLaunchKernelGGL((attn_fused_kernel<LP, 2>), dim3((num_heads + 7) & ~7, 2), dim3(1024), lds, ctx->stream, output, att, q,
-                           key_cache, value_cache, num_heads, head_size, kv_mul, row_stride, alpha, pos);
+                           key_cache, value_cache, num_heads, head_size, kv_mul, row_stride, alpha, pos, max_seq_len);
         return awq_check_launch("attn_fused");
     }
     hipLaunchKernelGGL((attn_scores_kernel<LP>), dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, ctx->stream, att, q,

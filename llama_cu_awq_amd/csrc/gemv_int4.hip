@@ -301,12 +301,6 @@ Int4Mat to_mat(const awq_qweight* w) { return Int4Mat{w->weight, w->zeros, w->sc
 
 bool qw_ok(const awq_qweight* w) { return w && w->weight && w->zeros && w->scales; }
 
-// Tuning overrides for experiments: AWQ_GEMV_WAVES, AWQ_GEMV_ROWS, AWQ_GEMV_DEPTH.
-int env_int(const char* name) {
-    const char* e = getenv(name);
-    return e ? atoi(e) : 0;
-}
-
 // Launch geometry of one matrix-vector product.
 struct GemvPlan {
     int waves;   // waves per workgroup (4, 8)
@@ -368,13 +362,7 @@ GemvPlan plan_for(int K, int rows) {
 
 template <int KIND, bool ROPE>
 int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan plan) {
-    static const int forced_w = env_int("AWQ_GEMV_WAVES");
-    static const int forced_r = env_int("AWQ_GEMV_ROWS");
-    static const int forced_d = env_int("AWQ_GEMV_DEPTH");
-    if (forced_w) plan.waves = forced_w;
-    if (forced_r) plan.rows = forced_r;
-    if (forced_d) plan.depth = forced_d;
-    if (p.norm_w && KIND == KIND_FFN && !forced_w && p.K <= 8192) plan.waves = 4;  // see launch()
+    if (p.norm_w && KIND == KIND_FFN && p.K <= 8192) plan.waves = 4;  // see launch()
     if (ROPE && plan.rows < 2) plan.rows = 2;  // a rotation pair lives in one wave
 #define AWQ_CASE(W_, R_) \
     if (plan.waves == W_ && plan.rows == R_) return dispatch_depth<W_, R_, KIND, ROPE>(ctx, p, grid_y, what, plan);
@@ -403,7 +391,6 @@ int awq_launch_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const
     p.pos = pos;
     p.norm_w = norm_w;
     p.norm_out = norm_out;
-    // 2 rows per wave keep >= 2 workgroups per CU busy at N = 4096; 4 rows amortise staging on big N
     return dispatch<KIND_SINGLE, false>(ctx, p, 1, "gemv_int4", plan_for(K, 1));
 }
 

@@ -877,6 +877,13 @@ int awq_launch_rope_rows(awq_ctx* ctx, uint16_t* q, uint16_t* kcache_layer, int 
     return awq_check_launch("rope_rows");
 }
 
+// Largest context (pos0 + M) the batched attention kernels take: they hold one fp16 score row per query in LDS.
+int awq_prefill_attention_max_positions(int head_size) {
+    const int lds_cap = 160 * 1024;
+    if (head_size == 128) return ((lds_cap - 2 * 128 * pf::VT_STRIDE * 2) / (pf::AQ * 2) - 8) & ~63;
+    return ((lds_cap - pf::BQ * head_size * 2 - pf::BQ * 8) / (pf::BQ * 2)) & ~7;
+}
+
 int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, const uint16_t* kc, const uint16_t* vc, int nh, int hs,
                             int kv_mul, int M, int pos0) {
     if (hs == 128) {

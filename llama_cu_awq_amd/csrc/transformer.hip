@@ -43,6 +43,7 @@ int awq_launch_rope_rows(awq_ctx* ctx, uint16_t* q, uint16_t* kcache_layer, int 
 int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, const uint16_t* kc, const uint16_t* vc, int nh, int hs,
                             int kv_mul, int M, int pos0);
 int awq_launch_set_pos(awq_ctx* ctx, int* pos_dev, volatile int* pos_host, int value);
+int awq_prefill_attention_max_positions(int head_size);
 int awq_launch_copy_row(awq_ctx* ctx, uint16_t* dst, const uint16_t* src, int n);
 
 namespace {
@@ -91,6 +92,10 @@ struct awq_transformer {
     std::vector<awq_layer_weights> layers;
     awq_run_state s;
     SharedData* shared;
+    // Position the next pass will run at, counted on the host as passes are ISSUED (the pinned copy in `shared` is
+    // only current after the stream has drained).  Sizes the attention launch, selects the graph bin and bounds
+    // the sequence; kept by reset / set_pos / forward / accept / sample / prefill.
+    int issued_pos;
     hipGraphExec_t graphs[2][kMaxGraphs];
     bool captured[2][kMaxGraphs];
     int* tokens_dev;  // device mirror of SharedData.tokens (the persistent kernel reads its input token here)
@@ -254,6 +259,7 @@ awq_transformer* new_transformer(awq_ctx* ctx) {
     t->tk_trace = nullptr;
     t->pf_rows = 0;
     t->pf_x = t->pf_xb = t->pf_q = t->pf_att = t->pf_hb = nullptr;
+    t->issued_pos = 0;
     memset(&t->s, 0, sizeof(t->s));
     memset(t->captured, 0, sizeof(t->captured));
     return t;
@@ -416,7 +422,6 @@ int plan_token_kernel(awq_transformer* t) {
     a.sync = t->tk_sync;
     a.err_host = t->tk_err_host;
     a.spin_limit = 50000000LL;  // 0.5 s of the 100 MHz wall clock
-    if (const char* e = getenv("AWQ_TK_SPIN_LIMIT")) a.spin_limit = atoll(e);
     a.lds_xs = 0;
     a.lds_ab = xs_bytes;
     a.lds_part = a.lds_ab + ab_bytes;
@@ -547,7 +552,11 @@ int awq_transformer_load_image(awq_ctx* ctx, const void* image, size_t bytes, aw
         release(t);
         return r;
     }
-    AWQ_HIP_TRY(hipDeviceSynchronize());
+    if (hipError_t e = hipDeviceSynchronize(); e != hipSuccess) {
+        awq_set_error("model set-up failed: %s", hipGetErrorString(e));
+        release(t);
+        return AWQ_ERR_HIP;
+    }
     *out = t;
     return AWQ_OK;
 }
@@ -630,7 +639,11 @@ int awq_transformer_load_file(awq_ctx* ctx, const char* checkpoint_path, awq_tra
         release(t);
         return r;
     }
-    AWQ_HIP_TRY(hipDeviceSynchronize());
+    if (hipError_t e = hipDeviceSynchronize(); e != hipSuccess) {
+        awq_set_error("model set-up failed: %s", hipGetErrorString(e));
+        release(t);
+        return AWQ_ERR_HIP;
+    }
     *out = t;
     return AWQ_OK;
 }
@@ -679,8 +692,11 @@ int awq_transformer_reset(awq_transformer* t, const int* prompt_tokens, int num_
     t->shared->pos = 0;
     memcpy(t->shared->tokens, prompt_tokens, sizeof(int) * (size_t)num_prompt_tokens);
     AWQ_HIP_TRY(hipMemcpy(t->tokens_dev, prompt_tokens, sizeof(int) * (size_t)num_prompt_tokens, hipMemcpyHostToDevice));
+    t->issued_pos = 0;
     if (t->tk_err_host) *t->tk_err_host = 0;
-    if (t->tk_sync) AWQ_HIP_TRY(hipMemset(&t->tk_sync->error, 0, sizeof(int)));
+    // After a barrier time-out the flag and release words hold epochs of a launch that never finished; start the
+    // persistent kernel's synchronisation state from scratch (all zero = the state of a fresh model).
+    if (t->tk_sync) AWQ_HIP_TRY(hipMemset(t->tk_sync, 0, sizeof(tk::Sync)));
     return AWQ_OK;
 }
 
@@ -693,6 +709,7 @@ int awq_transformer_set_pos(awq_transformer* t, int pos, int token) {
     t->shared->pos = pos;
     t->shared->tokens[pos] = token;
     AWQ_HIP_TRY(hipMemcpy(t->tokens_dev + pos, &token, sizeof(int), hipMemcpyHostToDevice));
+    t->issued_pos = pos;
     return AWQ_OK;
 }
 
@@ -711,22 +728,36 @@ int awq_transformer_prefill(awq_transformer* t, int n_tokens, int gen_token) {
         awq_set_error("prefill needs dim, kv_dim and hidden_dim to be multiples of 128 (got %d, %d, %d)", dim, kv_dim, hidden);
         return AWQ_ERR_SHAPE;
     }
-    AWQ_HIP_TRY(hipStreamSynchronize(ctx->stream));  // the host's view of the position must be current
-    const int pos_start = t->shared->pos;
+    const int pos_start = t->issued_pos;
     AWQ_REQUIRE(pos_start + n_tokens <= p.seq_len, AWQ_ERR_ARG, "prompt runs past seq_len");
+    // The batched attention keeps a score row per query in LDS, which bounds the context it can take; tokens past
+    // that bound go through the matrix-vector path one at a time (the definition of what prefill must leave behind).
+    const int max_ctx = awq_prefill_attention_max_positions(hs);
+    int n_batched = max_ctx - pos_start;
+    if (n_batched > n_tokens) n_batched = n_tokens;
+    if (n_batched < 0) n_batched = 0;
     const int chunk = 512;
-    if (t->pf_rows == 0) {
+    if (n_batched > 0 && t->pf_rows == 0) {
         const int rows = p.seq_len < chunk ? p.seq_len : chunk;
-        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_x, (size_t)rows * dim * 2));
-        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_xb, (size_t)rows * dim * 2));
-        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_q, (size_t)rows * dim * 2));
-        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_att, (size_t)rows * dim * 2));
-        AWQ_HIP_TRY(hipMalloc((void**)&t->pf_hb, (size_t)rows * hidden * 2));
+        uint16_t** bufs[5] = {&t->pf_x, &t->pf_xb, &t->pf_q, &t->pf_att, &t->pf_hb};
+        const size_t widths[5] = {(size_t)dim, (size_t)dim, (size_t)dim, (size_t)dim, (size_t)hidden};
+        for (int i = 0; i < 5; i++) {
+            hipError_t e = hipMalloc((void**)bufs[i], (size_t)rows * widths[i] * 2);
+            if (e != hipSuccess) {  // leave no half-allocated workspace behind
+                for (int j = 0; j < i; j++) {
+                    (void)hipFree(*bufs[j]);
+                    *bufs[j] = nullptr;
+                }
+                *bufs[i] = nullptr;
+                awq_set_error("prefill workspace allocation failed: %s", hipGetErrorString(e));
+                return AWQ_ERR_HIP;
+            }
+        }
         t->pf_rows = rows;
     }
     int r;
-    for (int done = 0; done < n_tokens; done += t->pf_rows) {
-        const int M = (n_tokens - done < t->pf_rows) ? n_tokens - done : t->pf_rows;
+    for (int done = 0; done < n_batched; done += t->pf_rows) {
+        const int M = (n_batched - done < t->pf_rows) ? n_batched - done : t->pf_rows;
         const int pos0 = pos_start + done;
         if ((r = awq_launch_embed_rows(ctx, t->pf_x, t->embed, dim, t->tokens_dev, pos0, M))) return r;
         for (int l = 0; l < p.n_layers; l++) {
@@ -759,6 +790,16 @@ int awq_transformer_prefill(awq_transformer* t, int n_tokens, int gen_token) {
                 return r;
         }
     }
+    if (n_batched < n_tokens) {
+        if (n_batched > 0 && (r = awq_launch_set_pos(ctx, t->s.pos, t->s.shared_pos, pos_start + n_batched))) return r;
+        for (int i = n_batched; i < n_tokens; i++) {
+            if ((r = network(t, pos_start + i + 1, AWQ_SCHEDULE_FUSED))) return r;
+            if ((r = awq_launch_argmax(ctx, t->s.logits, p.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos,
+                                       i == n_tokens - 1 ? gen_token : 0, t->tokens_dev)))
+                return r;
+        }
+    }
+    t->issued_pos = pos_start + n_tokens;
     return AWQ_OK;
 }
 
@@ -780,8 +821,6 @@ int awq_transformer_trace(awq_transformer* t, int enable, long long* host_out, i
         AWQ_HIP_TRY(hipStreamSynchronize(t->ctx->stream));
         AWQ_HIP_TRY(hipFree(t->tk_trace));
         t->tk_trace = nullptr;
-    t->pf_rows = 0;
-    t->pf_x = t->pf_xb = t->pf_q = t->pf_att = t->pf_hb = nullptr;
     }
     return AWQ_OK;
 }
@@ -793,7 +832,7 @@ int awq_transformer_forward_logits(awq_transformer* t, int use_graph, int mode) 
     (void)use_graph;  // the recorded sequences include the sampler; this entry point always launches eagerly
     awq_ctx* ctx = t->ctx;
     if (int r = awq_bind(ctx)) return r;
-    const int seq_len = t->shared->pos + 1;
+    const int seq_len = t->issued_pos + 1;
     AWQ_REQUIRE(seq_len <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
     return network(t, seq_len, mode);
 }
@@ -803,18 +842,22 @@ int awq_transformer_accept(awq_transformer* t, int token, int write_token) {
     AWQ_REQUIRE(token >= 0 && token < t->cfg.vocab_size, AWQ_ERR_ARG, "token out of range");
     awq_ctx* ctx = t->ctx;
     if (int r = awq_bind(ctx)) return r;
-    AWQ_REQUIRE(t->shared->pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+    AWQ_REQUIRE(t->issued_pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
     hipLaunchKernelGGL(accept_kernel, dim3(1), dim3(1), 0, ctx->stream, token, t->s.shared_tokens, t->tokens_dev, t->s.shared_pos,
                        t->s.pos, write_token);
-    return awq_check_launch("accept");
+    if (int r = awq_check_launch("accept")) return r;
+    t->issued_pos++;
+    return AWQ_OK;
 }
 
 int awq_transformer_sample(awq_transformer* t, awq_sampler* sampler, int gen_token) {
     AWQ_REQUIRE(t && sampler, AWQ_ERR_ARG, "null transformer or sampler");
     awq_ctx* ctx = t->ctx;
     if (int r = awq_bind(ctx)) return r;
-    AWQ_REQUIRE(t->shared->pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
-    return awq_sampler_run(sampler, t->s.logits, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token, t->tokens_dev);
+    AWQ_REQUIRE(t->issued_pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+    if (int r = awq_sampler_run(sampler, t->s.logits, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token, t->tokens_dev)) return r;
+    t->issued_pos++;
+    return AWQ_OK;
 }
 
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode) {
@@ -832,14 +875,17 @@ int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, in
             awq_set_error("persistent kernel: a grid barrier timed out (workgroups not co-resident?)");
             return AWQ_ERR_HIP;
         }
-        AWQ_REQUIRE(t->shared->pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+        AWQ_REQUIRE(t->issued_pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
         tk::Args a = t->tk_args;
         a.write_token = gen_token;
         a.trace = t->tk_trace;
-        return tk_launch(ctx->stream, a, t->tk_lds_bytes);
+        if (int r = tk_launch(ctx->stream, a, t->tk_lds_bytes)) return r;
+        t->issued_pos++;
+        return AWQ_OK;
     }
-    // llama2_q4.cu:552: the host's view of the position sizes the attention launch
-    const int seq_len = t->shared->pos + 1;
+    // llama2_q4.cu:552 sizes the attention launch from the pinned position after a synchronisation; the count of
+    // issued passes is the same number and does not need one
+    const int seq_len = t->issued_pos + 1;
     AWQ_REQUIRE(seq_len <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
     int r;
     if (use_graph) {
@@ -872,6 +918,7 @@ int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, in
         // token must survive, so those steps run eagerly below.
         if (gen_token) {
             AWQ_HIP_TRY(hipGraphLaunch(t->graphs[mode][graph_index], ctx->stream));
+            t->issued_pos++;
             return AWQ_OK;
         }
         r = network(t, seq_len_bin, mode);
@@ -879,7 +926,11 @@ int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, in
         r = network(t, seq_len, mode);
     }
     if (r) return r;
-    return awq_launch_argmax(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token, t->tokens_dev);
+    if ((r = awq_launch_argmax(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token,
+                               t->tokens_dev)))
+        return r;
+    t->issued_pos++;
+    return AWQ_OK;
 }
 
 }  // extern "C"

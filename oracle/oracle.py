@@ -188,6 +188,10 @@ class Model:
     def set_pos(self, pos, token):
         lib.orc_model_set_pos(self.h, pos, token)
 
+    @property
+    def pos(self):
+        return lib.orc_model_pos(self.h)
+
     def forward(self, gen_token=True):
         return lib.orc_model_forward(self.h, int(gen_token))
 

@@ -215,7 +215,9 @@ def test_attention_brute_force(heads, head, kv_mul, pos):
         assert np.allclose(att[h].astype(np.float64), p, atol=2e-3)
         assert abs(att[h].astype(np.float64).sum() - 1) <= 5e-3
     if pos == 0:
-        assert np.array_equal(out.view(np.uint16), np.tile(vc.view(np.uint16).reshape(heads // kv_mul, head), (1, kv_mul)).reshape(-1)) or kv_mul > 1
+        # one position: probability 1, so every head returns its KV head's value row bit for bit
+        want = np.repeat(vc.view(np.uint16).reshape(heads // kv_mul, head), kv_mul, axis=0).reshape(-1)
+        assert np.array_equal(out.view(np.uint16), want)
 
 
 def test_attention_identical_keys_give_uniform_probabilities():

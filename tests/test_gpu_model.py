@@ -45,7 +45,8 @@ def test_one_token_state(pair, mode):
         t.forward(gen_token=False, use_graph=False, mode=mode)
         o.forward(gen_token=False)
     t.ctx.sync()
-    assert t.pos == 3 == o.tokens(0) or t.pos == 3
+    assert t.pos == 3 and o.pos == 3
+    assert [t.token(i) for i in range(4)] == prompt == o.tokens(4)  # prompt steps leave the token list alone
     kv_dim = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"]
     for name, n in (("logits", cfg["vocab_size"]), ("hb", cfg["hidden_dim"]), ("q", cfg["dim"]), ("key_cache", 3 * kv_dim), ("value_cache", 3 * kv_dim)):
         got = f16(t.download(name, n))

@@ -124,7 +124,6 @@ def test_qkv_matvec(ctx, K, N):
     oracle.qkv_matvec(q, kc, vc, x, *mats, K, N, loff, pos)
     for got, want in ((dq.download(np.uint16), q), (dk.download(np.uint16), kc), (dv.download(np.uint16), vc)):
         assert_close_f16(f16(got), f16(want), ulps=2)
-        assert np.array_equal(got == 0, want == 0) or True
     # only the addressed cache row is written
     kgot = dk.download(np.uint16)
     assert not kgot[: loff + pos * N].any() and not kgot[loff + (pos + 1) * N :].any()
