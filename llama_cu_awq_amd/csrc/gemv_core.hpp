@@ -15,31 +15,30 @@ struct XArgs {
     int C;                   // 32-element chunks = ceil(K / 32)
 };
 
-// sum over the 32 consecutive K elements of one chunk of (q - z) * x.
+// 2^-24 * sum over the 32 consecutive K elements of one chunk of (q - z) * x.
 //
 // w: 4 dwords of 8 nibbles.  xq[qi]: the 8 activations of dword qi as fp16 pairs
-// (x0,x4) (x1/16,x5/16) (x2,x6) (x3/16,x7/16).  OR-ing a nibble into the
-// mantissa of fp16 1024.0 gives 1024+q (nibble at bits 0-3) or 1024+16q (bits
-// 4-7) exactly, so
-//   sum_k (1024 + [16] q_k) * X_k  =  1024 * sum_k X_k  +  sum_k q_k x_k
-// and the chunk's constants A = sum x and B = 1024 * sum X (computed once when
-// x is staged) turn that into sum (q - z) x = dot - B - z*A.  The accumulator
-// starts at -B - z*A so that the large common term cancels first.  Products are
-// exact in fp32 (11-bit x 11-bit significands); only the fp32 additions round.
-__device__ __forceinline__ float chunk_dot(const u32x4 w, const float zf, const u32x4 (&xq)[4], const float A, const float B,
-                                           const uint32_t magic) {
-    float acc = fmaf(-zf, A, -B);
+// (x0,x4) (x1/16,x5/16) (x2,x6) (x3/16,x7/16).  A nibble masked out in place IS an fp16 number: with sign and
+// exponent bits zero, the bit pattern 0x000q is the denormal q * 2^-24 and 0x00q0 is 16q * 2^-24, both exact, and
+// v_dot2_f32_f16 takes denormal inputs at face value.  So each masked dword half multiplies its activation without
+// any offset to cancel: the products (at most 4 x 11 significant bits) are exact in fp32, and only the fp32
+// additions round, at the magnitude of the result itself (the reference adds fp32 products (q - z) * s * x the same
+// way, gpu_kernels.h:204-206).  The zero point comes in through the chunk's constant A = 2^-24 * sum x (computed
+// once when x is staged): the accumulator starts at -z * A.  The caller multiplies the result by 2^24 * scale.
+__device__ __forceinline__ float chunk_dot(const u32x4 w, const float zf, const u32x4 (&xq)[4], const float A) {
+    float acc = -zf * A;
 #pragma unroll
     for (int qi = 0; qi < 4; qi++) {
         const uint32_t d = w[qi];
         const uint32_t d8 = d >> 8;
-        acc = dot2((d & 0x000F000Fu) | magic, xq[qi][0], acc);
-        acc = dot2((d & 0x00F000F0u) | magic, xq[qi][1], acc);
-        acc = dot2((d8 & 0x000F000Fu) | magic, xq[qi][2], acc);
-        acc = dot2((d8 & 0x00F000F0u) | magic, xq[qi][3], acc);
+        acc = dot2(d & 0x000F000Fu, xq[qi][0], acc);
+        acc = dot2(d & 0x00F000F0u, xq[qi][1], acc);
+        acc = dot2(d8 & 0x000F000Fu, xq[qi][2], acc);
+        acc = dot2(d8 & 0x00F000F0u, xq[qi][3], acc);
     }
     return acc;
 }
+constexpr float kChunkDotUnscale = 16777216.0f;  // 2^24
 
 // One 64-lane pass over the NS row streams of a wave: 16 bytes of packed weights per lane and stream, the zero-point
 // dword and the scale that cover them, and (residual form) the value the result is added to.
@@ -52,7 +51,7 @@ struct Stage {
 };
 
 // Staging of x (K halves) into LDS: xs[qi*C + c] holds the 8 activations of dword qi of chunk c as pairs
-// (x0,x4)(x1/16,x5/16)(x2,x6)(x3/16,x7/16), and ab[c] = {A, B} the chunk constants described at chunk_dot.  Elements
+// (x0,x4)(x1/16,x5/16)(x2,x6)(x3/16,x7/16), and ca[c] the chunk constant A described at chunk_dot.  Elements
 // in [K, 32*C) are zero.  With NORM the vector is RMS-normalised on the way in with the reference's arithmetic
 // (gpu_kernels.h:72-105): o = half(x * (rsqrt(mean(x^2) + 1e-5) * w)).
 //
@@ -84,7 +83,7 @@ __device__ __forceinline__ void load_x(XPieces<NORM>& xr, const XArgs& p) {
 
 // One piece of 8 halves: normalise (optional), permute, reduce the chunk constants over the 4 lanes of a chunk, store.
 template <bool NORM>
-__device__ __forceinline__ void stage_piece(u32x4* xs, float2* ab, const XArgs& p, int e, u32x4 v, u32x4 wv, float ss,
+__device__ __forceinline__ void stage_piece(u32x4* xs, float* ca, const XArgs& p, int e, u32x4 v, u32x4 wv, float ss,
                                             bool store_norm) {
     const int n8 = p.K >> 3;
     if (e >= n8) v = u32x4{0u, 0u, 0u, 0u};
@@ -115,16 +114,13 @@ __device__ __forceinline__ void stage_piece(u32x4* xs, float2* ab, const XArgs& 
     const float even = dot2(as_u32(p0), ones, dot2(as_u32(p2), ones, 0.0f));
     const float odd = dot2(as_u32(p1), ones, dot2(as_u32(p3), ones, 0.0f));
     float a = fmaf(16.0f, odd, even);  // sum of the activations as the dot product sees them
-    float b = even + odd;              // sum of the stored fp16 values
     // the 4 dword pieces of a chunk sit in 4 adjacent lanes
     a += dpp_mov<0xB1>(a);
     a += dpp_mov<0x4E>(a);
-    b += dpp_mov<0xB1>(b);
-    b += dpp_mov<0x4E>(b);
     if (e < p.C * 4) {
         u32x4 o = {as_u32(p0), as_u32(p1), as_u32(p2), as_u32(p3)};
         xs[(e & 3) * p.C + (e >> 2)] = o;
-        if ((e & 3) == 0) ab[e >> 2] = make_float2(a, 1024.0f * b);
+        if ((e & 3) == 0) ca[e >> 2] = a * (1.0f / kChunkDotUnscale);
     }
 }
 
@@ -141,7 +137,7 @@ __device__ __forceinline__ float piece_sumsq(u32x4 v, float part) {
 
 // red: W + 1 floats of LDS.
 template <int W, bool NORM>
-__device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const XArgs& p, float* red, const XPieces<NORM>& xr) {
+__device__ __forceinline__ void stage_x(u32x4* xs, float* ca, const XArgs& p, float* red, const XPieces<NORM>& xr) {
     constexpr int T = W * 64;
     const int tid = threadIdx.x;
     const int n8 = p.K >> 3;
@@ -180,14 +176,14 @@ __device__ __forceinline__ void stage_x(u32x4* xs, float2* ab, const XArgs& p, f
 #pragma unroll
     for (int i = 0; i < XP; i++)
         if (i * T < p.C * 4)  // uniform: the quad reduction needs all lanes
-            stage_piece<NORM>(xs, ab, p, i * T + tid, xr.v[i], xr.w[NORM ? i : 0], ss, store_norm);
+            stage_piece<NORM>(xs, ca, p, i * T + tid, xr.v[i], xr.w[NORM ? i : 0], ss, store_norm);
     for (int e0 = XP * T; e0 < p.C * 4; e0 += T) {
         const int e = e0 + tid;
         const int ec = min(e, n8 - 1);
         const u32x4 v = xg[ec];
         u32x4 wv = v;
         if (NORM) wv = wg[ec];
-        stage_piece<NORM>(xs, ab, p, e, v, wv, ss, store_norm);
+        stage_piece<NORM>(xs, ca, p, e, v, wv, ss, store_norm);
     }
     __syncthreads();
 }

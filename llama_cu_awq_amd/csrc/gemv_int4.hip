@@ -12,9 +12,9 @@
 // Each wave owns R consecutive rows (one gate/up pair in the fused FFN form) and walks them in passes of 64 x 16
 // bytes with D passes in flight.  Loads return in order, so a wave first requests its share of the activations,
 // then its first D passes of weights, and stages the activations while the weights are still on their way.
-// Nibbles become fp16 numbers by OR-ing them into the mantissa of 1024.0, products are accumulated in fp32 by
-// v_dot2_f32_f16 with the 1024 offset and the zero point cancelled through per-chunk constants, and the group scale
-// is applied once per 32 elements.
+// Nibbles are used in place as fp16 denormals (q * 2^-24: a mask is the whole conversion), products are accumulated
+// in fp32 by v_dot2_f32_f16, the zero point enters through a per-chunk constant, and the group scale (times 2^24) is
+// applied once per 32 elements.
 #include <math.h>
 #include <stdlib.h>
 
@@ -69,12 +69,10 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     const int C = p.C;
     const int pwh = C * 4;
     const int P = (C + 63) >> 6;  // 64-lane passes per row
-    float2* ab = reinterpret_cast<float2*>(xs + 4 * C);
+    float* ca = reinterpret_cast<float*>(xs + 4 * C);
     const int which = (KIND == KIND_QKV) ? blockIdx.y : 0;
     const bool rope_here = ROPE && which != 2;
     constexpr bool RES = KIND == KIND_SINGLE;
-    uint32_t magic = 0x64006400u;  // fp16 pair (1024.0, 1024.0), kept in a VGPR
-    asm("" : "+v"(magic));
 
     constexpr int NS = (KIND == KIND_FFN) ? 2 * R : R;
     const Int4Mat m0 = (KIND == KIND_QKV) ? (which == 0 ? p.m[0] : (which == 1 ? p.m[1] : p.m[2])) : p.m[0];
@@ -154,7 +152,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     int cg = g_begin, cp = 0, cs = 0;
     auto finish_group = [&](const Stage<NS>& st) {
 #pragma unroll
-        for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]);
+        for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]) * kChunkDotUnscale;  // chunk_dot works in units of 2^-24
         const int li0 = (cg * W + wave) * R;
         if (lane == 0 && li0 < p.N) {
             if (rope_here) {
@@ -203,12 +201,12 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
             u32x4 xq[4];
 #pragma unroll
             for (int qi = 0; qi < 4; qi++) xq[qi] = xs[qi * C + cc];
-            const float2 cab = ab[cc];
+            const float cA = ca[cc];
             const int zshift = ((cc >> 2) & 7) * 4;
 #pragma unroll
             for (int i = 0; i < NS; i++) {
                 const float zf = (float)((st.zw[i] >> zshift) & 0xFu);
-                const float acc = chunk_dot(st.w[i], zf, xq, cab.x, cab.y, magic);
+                const float acc = chunk_dot(st.w[i], zf, xq, cA);
                 const float sc = c < C ? half_bits_to_float(st.s[i]) : 0.0f;
                 sum[i] = fmaf(sc, acc, sum[i]);
             }
@@ -231,7 +229,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     set_rows(lg);
 #pragma unroll
     for (int d = 0; d < D; d++) issue(st[d]);
-    stage_x<W, NORM>(xs, ab, xa, red, xr);
+    stage_x<W, NORM>(xs, ca, xa, red, xr);
     const int rounds = (total + D - 1) / D;
     for (int r = 1; r < rounds; r++) {
 #pragma unroll
@@ -327,7 +325,7 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
         if (gx > 3 * cus) gx = 3 * cus;
     }
     const dim3 grid(gx, grid_y);
-    const size_t lds = (size_t)p.C * 72;  // activations + per-chunk constants
+    const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
     if (p.norm_w)
         hipLaunchKernelGGL((gemv_int4_kernel<W, R, D, KIND, true, ROPE>), grid, dim3(W * 64), lds, ctx->stream, p);
     else

@@ -94,8 +94,10 @@ def unpack_nibbles(packed, n):
     return ((packed[:, :, None] >> shifts) & np.uint32(0xF)).reshape(rows, width * 8)[:, :n].astype(np.uint8)
 
 
-def make_qweight(key, K, N):
-    """Random packed matrix: returns (weight (N,pwh) u32, zeros (N,pzh) u32, scales (N,sh) f16)."""
+def make_qweight(key, K, N, scale_mult=1.0):
+    """Random packed matrix: returns (weight (N,pwh) u32, zeros (N,pzh) u32, scales (N,sh) f16).
+
+    scale_mult multiplies the scale range U[0.002, 0.02] (1.0 = the benchmark distribution)."""
     pwh, pzh, sh = strides(K)
     weight = random_u32(stream_key(key, "w"), N * pwh).reshape(N, pwh).copy()
     if K % 32:
@@ -103,7 +105,7 @@ def make_qweight(key, K, N):
         weight = pack_nibbles(q, pwh)
     z = (random_u64(stream_key(key, "z"), N * sh) >> np.uint64(60)).astype(np.uint32).reshape(N, sh)
     zeros = pack_nibbles(z, pzh)
-    scales = (0.002 + 0.018 * uniform01(stream_key(key, "s"), N * sh)).astype(np.float16).reshape(N, sh)
+    scales = (scale_mult * (0.002 + 0.018 * uniform01(stream_key(key, "s"), N * sh))).astype(np.float16).reshape(N, sh)
     return weight, zeros, scales
 
 
@@ -131,8 +133,12 @@ def model_bytes(cfg):
     return 32 + 4 * V * dim + 2 * dim + L * layer
 
 
-def make_model_image(cfg, seed=0, threads=8):
-    """A weight_packer-format .bin image (llama2_q4.cu:220-246 order) of random weights, as a uint8 array."""
+def make_model_image(cfg, seed=0, threads=8, scale_mult=1.0):
+    """A weight_packer-format .bin image (llama2_q4.cu:220-246 order) of random weights, as a uint8 array.
+
+    scale_mult shrinks (or grows) every quantisation scale: with the benchmark distribution (1.0) each layer adds a
+    few hundred to the residual stream, which leaves fp16 range in models of 40 and more layers; a smaller range
+    keeps such a model finite so that its outputs can be checked."""
     dim, hid, L, V = cfg["dim"], cfg["hidden_dim"], cfg["n_layers"], cfg["vocab_size"]
     kv_dim = dim * cfg["n_kv_heads"] // cfg["n_heads"]
     img = np.empty(model_bytes(cfg), dtype=np.uint8)
@@ -153,7 +159,7 @@ def make_model_image(cfg, seed=0, threads=8):
         pwh, pzh, sh = strides(K)
 
         def gen():
-            w, z, s = make_qweight(stream_key(seed, layer, name), K, N)
+            w, z, s = make_qweight(stream_key(seed, layer, name), K, N, scale_mult)
             return np.concatenate([w.reshape(-1).view(np.uint8), z.reshape(-1).view(np.uint8), s.reshape(-1).view(np.uint8)])
 
         put(N * (pwh * 4 + pzh * 4 + sh * 2), gen)

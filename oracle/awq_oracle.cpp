@@ -156,12 +156,19 @@ void orc_dequant(uint16_t* out, const uint32_t* weight, const uint32_t* zeros, c
 }
 
 // ---------------------------------------------------------------- int4 dot
+// Diagnostic switch (off by default): matrix-vector sums in double precision instead of the reference's fp32 order.
+static int g_exact_sums = 0;
+extern "C" void orc_set_exact_sums(int on) { g_exact_sums = on; }
+
 // One output row of the fused unpack/dequant/dot, with the reference's
 // lane structure: 32 lanes, lane L owns the uint4 (32 consecutive K
 // elements) at dword ygq*128 + L*4 of each 1024-element tile; fp32
 // w = (q - z) * scale; sum = fma(w, x, sum); then a shuffle-down tree over the
 // 32 lane sums (gpu_kernels.h:179-218).
+static float row_dot_int4_exact(int index, const h16* x, const QW& m, int K, int pzh, int sh, int pwh);
+
 static float row_dot_int4(int index, const h16* x, const QW& m, int K, int pzh, int sh, int pwh) {
+    if (g_exact_sums) return row_dot_int4_exact(index, x, m, K, pzh, sh, pwh);
     float lane_sum[32];
     for (int lane = 0; lane < 32; lane++) {
         float sum = 0.0f;
@@ -190,6 +197,20 @@ static float row_dot_int4(int index, const h16* x, const QW& m, int K, int pzh, 
     for (int off = 16; off > 0; off >>= 1)
         for (int i = 0; i < off; i++) lane_sum[i] += lane_sum[i + off];
     return lane_sum[0];
+}
+
+// The same row with every product and sum in double precision, rounded to fp32 once: the value that any fp32
+// summation order approximates.  Used only to measure how far the reference's own summation order is from it.
+static float row_dot_int4_exact(int index, const h16* x, const QW& m, int K, int pzh, int sh, int pwh) {
+    (void)pwh;
+    double sum = 0.0;
+    for (int k = 0; k < K; k++) {
+        const int g = k >> 7;
+        const double q = (double)((m.weight[(size_t)index * pwh + (k >> 3)] >> (4 * (k & 7))) & 0xFu);
+        const double z = (double)((m.zeros[(size_t)index * pzh + (g >> 3)] >> (4 * (g & 7))) & 0xFu);
+        sum += (q - z) * (double)h2f(m.scales[(size_t)index * sh + g]) * (double)h2f(x[k]);
+    }
+    return (float)sum;
 }
 
 // out = half(W x [+ out/gpu_count]), optionally written at out + loff + pos*N
@@ -304,6 +325,12 @@ int orc_matvec_f16(uint16_t* out, const uint16_t* x, const uint16_t* w, int n, i
     int serialLoads = div_up(div_up(n, 32), 8);
 #pragma omp parallel for schedule(static)
     for (int index = 0; index < d; index++) {
+        if (g_exact_sums) {
+            double acc = 0.0;
+            for (int j = 0; j < n; j++) acc += (double)h2f(w[(size_t)index * n + j]) * (double)h2f(x[j]);
+            out[index] = f2h((float)acc);
+            continue;
+        }
         float lane_sum[32];
         for (int lane = 0; lane < 32; lane++) {
             float sum = 0.0f;

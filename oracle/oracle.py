@@ -27,6 +27,7 @@ def _load():
         "orc_half_to_float": ([C.c_uint16], f),
         "orc_float_to_half": ([f], C.c_uint16),
         "orc_num_threads": ([], i),
+        "orc_set_exact_sums": ([i], None),
         "orc_dequant": ([vp, vp, vp, vp, i, i], None),
         "orc_matvec_int4": ([vp, vp, vp, vp, vp, i, i, i, i, i, vp], i),
         "orc_qkv_matvec": ([vp] * 13 + [i, i, i, vp], i),
@@ -72,6 +73,12 @@ def _c(a, dtype):
 
 def num_threads():
     return lib.orc_num_threads()
+
+
+def set_exact_sums(on):
+    """Diagnostic: matrix-vector sums in double precision (rounded to fp32 once) instead of the reference's fp32 order.
+    Process-wide; switch it off again after use."""
+    lib.orc_set_exact_sums(int(on))
 
 
 def dequant(weight, zeros, scales, K, N):

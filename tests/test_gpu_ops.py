@@ -93,7 +93,9 @@ def test_matvec_int4_accum_and_kv_offset(ctx):
 
 
 def test_zero_weights_leave_residual(ctx):
-    """accum with W == 0 (q == z everywhere) returns the residual unchanged."""
+    """accum with W == 0 (q == z everywhere) returns the residual.  The kernel forms sum q*x - z * sum x with each sum
+    rounded in fp32 on its own, so W x comes out as fp32 rounding noise (around 1e-7 here) instead of an exact zero:
+    the residual comes back bit for bit except where that noise crosses an fp16 rounding boundary (one step)."""
     K, N = 256, 64
     pwh, pzh, sh = synth.strides(K)
     w = np.full((N, pwh), 0x55555555, dtype=np.uint32)
@@ -104,7 +106,13 @@ def test_zero_weights_leave_residual(ctx):
     qw = A.QWeight.upload(ctx, w, z, s)
     dout = ctx.upload(resid)
     A.matmul_q(ctx, dout, ctx.upload(x), qw, K, N, accum=True)
-    assert np.array_equal(dout.download(np.uint16), resid.view(np.uint16))
+    got = dout.download(np.uint16)
+    steps = ulp_diff_f16(f16(got), resid)
+    assert steps.max() <= 1 and (steps == 0).mean() >= 0.9
+    # W x itself: zero to within fp32 rounding of its two partial sums
+    dout = ctx.zeros(N * 2)
+    A.matmul_q(ctx, dout, ctx.upload(x), qw, K, N)
+    assert np.abs(f16(dout.download(np.uint16)).astype(np.float64)).max() <= 1e-5
 
 
 @pytest.mark.parametrize("K,N", [(4096, 4096), (5120, 5120), (256, 64)])
