@@ -247,6 +247,17 @@ int awq_transformer_sample(awq_transformer* t, awq_sampler* sampler, int gen_tok
 int awq_gemm_int4(awq_ctx* ctx, uint16_t* out, int ldo, const uint16_t* a, int lda, int M, const awq_qweight* w, int K, int N,
                   int accum);
 
+/* awq_gemm_int4 for callers that cannot allocate device memory (code recorded into a HIP graph, serving loops and
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, shapes and results as
+ * awq_gemm_int4; the workspace of the split-K form (matrices with fewer than 256 output tiles of 128 x 128: fp32
+ * partial tiles and arrival counters, up to 32 MiB) lives in a device array inside the library instead of being
+ * allocated on first use, so this call makes no hipMalloc / hipFree and configures nothing (that happens per device
+ * when a context is created).  All calls on one GPU share that array: calls that overlap on one GPU (two streams,
+ * two contexts) race and must be serialised by the caller; calls on one stream are safe.  A shape whose split form
+ * would need more tiles than the array holds is refused with AWQ_ERR_SHAPE. */
+int awq_gemm_int4_static(awq_ctx* ctx, uint16_t* out, int ldo, const uint16_t* a, int lda, int M, const awq_qweight* w, int K,
+                         int N, int accum);
+
 /* Consume the n_tokens tokens at positions pos .. pos+n_tokens-1 of the shared token list in one batched pass:
  * afterwards the KV cache rows, the logits (of the last token), the token list and the position are those that
  * n_tokens calls of awq_transformer_forward (gen_token false for all but the last, `gen_token` for the last) would

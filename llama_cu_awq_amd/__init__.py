@@ -12,6 +12,7 @@ from .ops import (  # noqa: F401
     dequant,
     ffn_matvec_silu,
     gemm_q,
+    gemm_q_static,
     matmul,
     matmul_q,
     qkv_matvec,

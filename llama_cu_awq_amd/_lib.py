@@ -80,6 +80,7 @@ PROTOTYPES = {
     "awq_transformer_set_pos": [_vp, _i, _i],
     "awq_transformer_forward": [_vp, _i, _i, _i],
     "awq_gemm_int4": [_vp, _vp, _i, _vp, _i, _i, _pq, _i, _i, _i],
+    "awq_gemm_int4_static": [_vp, _vp, _i, _vp, _i, _i, _pq, _i, _i, _i],
     "awq_transformer_prefill": [_vp, _i, _i],
     "awq_transformer_forward_logits": [_vp, _i, _i],
     "awq_transformer_accept": [_vp, _i, _i],

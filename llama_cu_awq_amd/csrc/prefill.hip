@@ -12,6 +12,8 @@
 // times the fp16 scale in one rounding.
 #include <string.h>
 
+#include <mutex>
+
 #include "common.hpp"
 
 typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
@@ -761,17 +763,65 @@ __global__ __launch_bounds__(256) void copy_row_kernel(uint16_t* dst, const uint
 
 }  // namespace pf
 
-// ---------------------------------------------------------------- launchers (internal)
-static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* what) {
-    static bool lds_raised = false;  // the kernel's 80 KB of LDS exceed the default dynamic limit
-    if (!lds_raised) {
+// ---------------------------------------------------------------- split-K workspace that needs no allocation
+// awq_gemm_int4_static keeps the split-K workspace (fp32 partial tiles, then the per-tile arrival counters) in this
+// file-scope device array instead of memory obtained with hipMalloc.  Every GPU the library runs on holds its own copy
+// at its own address until the process ends.  In host code the array's name is only a stand-in for the symbol: the
+// device address is looked up once per device with hipGetSymbolAddress and kept in g_scratch_ptr, and that pointer is
+// what kernels and clears receive.
+constexpr int kStaticTiles = 256;  // the split form is taken below 256 tiles only
+constexpr size_t kStaticPartBytes = (size_t)kStaticTiles * 2 * pf::BM * pf::BN * sizeof(float);  // 32 MiB
+constexpr size_t kStaticScratchBytes = kStaticPartBytes + kStaticTiles * sizeof(unsigned int);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices];    // device address of `scratch` on each device, null until looked up
+static bool g_gemm_lds_raised[kMaxDevices];  // the GEMM kernel's dynamic LDS limit has been raised on the device
+
+namespace pf {
+__global__ void clear_words_kernel(unsigned int* words, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) words[i] = 0u;
+}
+}  // namespace pf
+
+// Once per device, with that device current: raise the GEMM kernel's LDS limit and look up the address of `scratch`.
+// Called when a context is created, so that the entry points themselves do no set-up work.
+int awq_gemm_device_setup(int device) {
+    if (device < 0 || device >= kMaxDevices) {
+        awq_set_error("device ordinal %d out of range", device);
+        return AWQ_ERR_ARG;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_gemm_lds_raised[device]) {
         hipError_t e = hipFuncSetAttribute((const void*)pf::gemm_int4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                            pf::GEMM_LDS_BYTES);
         if (e != hipSuccess) {
             awq_set_error("hipFuncSetAttribute(gemm_int4) failed: %s", hipGetErrorString(e));
             return AWQ_ERR_HIP;
         }
-        lds_raised = true;
+        g_gemm_lds_raised[device] = true;
+    }
+    if (!g_scratch_ptr[device]) {
+        void* ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            awq_set_error("hipGetSymbolAddress(scratch) failed on device %d: %s", device, hipGetErrorString(e));
+            return AWQ_ERR_HIP;
+        }
+        g_scratch_ptr[device] = ptr;
+    }
+    return AWQ_OK;
+}
+
+// ---------------------------------------------------------------- launchers (internal)
+// static_ws: take the split-K workspace from the file-scope device array (no allocation) instead of the context's.
+static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* what, bool static_ws = false) {
+    // the kernel's 80 KB of LDS exceed the default dynamic limit; raised per device when a context is created
+    // (contexts on a caller's stream included), here only for a device that was missed
+    if (ctx->device < 0 || ctx->device >= kMaxDevices || !g_gemm_lds_raised[ctx->device]) {
+        if (int r = awq_gemm_device_setup(ctx->device)) return r;
     }
     if ((size_t)p.M * (size_t)p.lda * 2 >= ((size_t)1 << 32)) {  // the kernel addresses A by 32-bit byte offsets
         awq_set_error("%s: activation block of %d x %d halves exceeds 4 GB", what, p.M, p.lda);
@@ -784,7 +834,26 @@ static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* 
     if ((p.epi == pf::EPI_STORE || p.epi == pf::EPI_RESID) && p.mtiles * ntiles < 256 && p.K >= 8 * pf::BK) {
         const size_t tiles = (size_t)p.mtiles * ntiles;
         const size_t need = tiles * 2 * pf::BM * pf::BN * sizeof(float);
-        if (ctx->gemm_part_bytes < need || ctx->gemm_counter_count < tiles) {
+        if (static_ws) {
+            if (tiles > (size_t)kStaticTiles) {
+                awq_set_error("%s: %zu output tiles of 128 x 128 exceed the %d the static split-K workspace holds", what, tiles,
+                              kStaticTiles);
+                return AWQ_ERR_SHAPE;
+            }
+            unsigned char* ws = static_cast<unsigned char*>(g_scratch_ptr[ctx->device]);
+            if (!ws) {
+                awq_set_error("%s: the static workspace was not set up on device %d", what, ctx->device);
+                return AWQ_ERR_HIP;
+            }
+            p.ksplit = 2;
+            p.part = reinterpret_cast<float*>(ws);
+            p.part_counter = reinterpret_cast<unsigned int*>(ws + kStaticPartBytes);
+            // the array keeps whatever the previous call on this GPU left: the arrival counters must start at zero
+            // (a fill kernel rather than a memset node, so that the call can be recorded into a graph)
+            hipLaunchKernelGGL(pf::clear_words_kernel, dim3(div_up((int)tiles, 256)), dim3(256), 0, ctx->stream, p.part_counter,
+                               (int)tiles);
+            if (int r = awq_check_launch("clear_words")) return r;
+        } else if (ctx->gemm_part_bytes < need || ctx->gemm_counter_count < tiles) {
             AWQ_HIP_TRY(hipStreamSynchronize(ctx->stream));
             if (ctx->gemm_part) (void)hipFree(ctx->gemm_part);
             if (ctx->gemm_counter) (void)hipFree(ctx->gemm_counter);
@@ -798,9 +867,11 @@ static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* 
             ctx->gemm_part_bytes = need;
             ctx->gemm_counter_count = tiles;
         }
-        p.ksplit = 2;
-        p.part = ctx->gemm_part;
-        p.part_counter = ctx->gemm_counter;
+        if (!static_ws) {
+            p.ksplit = 2;
+            p.part = ctx->gemm_part;
+            p.part_counter = ctx->gemm_counter;
+        }
     }
     // ids go round-robin over the 8 XCDs; each XCD takes every 8th weight tile with all of its M tiles (and K halves)
     const int grid = 8 * p.mtiles * p.ksplit * div_up(ntiles, 8);
@@ -831,11 +902,11 @@ static void gemm_common(pf::GemmParams& p, const uint16_t* A, int lda, int M, in
 }
 
 int awq_launch_gemm_single(awq_ctx* ctx, uint16_t* out, long long ldo, const uint16_t* A, int lda, int M, const awq_qweight* w,
-                           int K, int N, int accum) {
+                           int K, int N, int accum, bool static_ws) {
     pf::GemmParams p;
     gemm_common(p, A, lda, M, K, accum ? pf::EPI_RESID : pf::EPI_STORE);
     set_mat(p, 0, w, N, out, ldo, 0);
-    return launch_gemm(ctx, p, N / pf::BN, "gemm_int4");
+    return launch_gemm(ctx, p, N / pf::BN, "gemm_int4", static_ws);
 }
 
 int awq_launch_gemm_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, long long kv_row0_off,
@@ -955,7 +1026,21 @@ int awq_gemm_int4(awq_ctx* ctx, uint16_t* out, int ldo, const uint16_t* a, int l
         awq_set_error("awq_gemm_int4: needs M > 0, K %% 32 == 0, N %% 128 == 0, lda %% 8 == 0 (got M=%d K=%d N=%d lda=%d)", M, K, N, lda);
         return AWQ_ERR_SHAPE;
     }
-    return awq_launch_gemm_single(ctx, out, ldo, a, lda, M, w, K, N, accum);
+    return awq_launch_gemm_single(ctx, out, ldo, a, lda, M, w, K, N, accum, false);
+}
+
+int awq_gemm_int4_static(awq_ctx* ctx, uint16_t* out, int ldo, const uint16_t* a, int lda, int M, const awq_qweight* w, int K,
+                         int N, int accum) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(out && a && w && w->weight && w->zeros && w->scales, AWQ_ERR_ARG, "null pointer");
+    if (M <= 0 || K <= 0 || N <= 0 || (K & 31) || (N & 127) || (lda & 7)) {
+        awq_set_error("awq_gemm_int4_static: needs M > 0, K %% 32 == 0, N %% 128 == 0, lda %% 8 == 0 (got M=%d K=%d N=%d lda=%d)", M, K, N,
+                      lda);
+        return AWQ_ERR_SHAPE;
+    }
+    AWQ_REQUIRE(ctx->device >= 0 && ctx->device < kMaxDevices && g_scratch_ptr[ctx->device] && g_gemm_lds_raised[ctx->device],
+                AWQ_ERR_HIP, "the static workspace was not set up on this device when the context was created");
+    return awq_launch_gemm_single(ctx, out, ldo, a, lda, M, w, K, N, accum, true);
 }
 
 }  // extern "C"

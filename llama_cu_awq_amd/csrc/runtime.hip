@@ -8,6 +8,8 @@
 
 #include "common.hpp"
 
+int awq_gemm_device_setup(int device);  // prefill.hip
+
 static std::mutex g_err_mutex;
 static char g_err[1024] = "";
 
@@ -51,7 +53,14 @@ int awq_device_info(int device, char* name, size_t name_bytes, size_t* global_me
     return AWQ_OK;
 }
 
+// The device is current when this runs.
 static int ctx_init(int device, hipStream_t stream, bool owns, awq_ctx** out) {
+    // per-device set-up of the batched GEMM (kernel attribute, address of its static workspace): done here so that
+    // the entry points themselves neither allocate nor configure anything
+    if (int r = awq_gemm_device_setup(device)) {
+        if (owns) (void)hipStreamDestroy(stream);
+        return r;
+    }
     awq_ctx* c = new awq_ctx();
     c->device = device;
     c->stream = stream;

@@ -30,7 +30,7 @@ int awq_sampler_run(awq_sampler* s, uint16_t* logits, int* tokens, volatile int*
                     int* mirror);
 // prefill.hip
 int awq_launch_gemm_single(awq_ctx* ctx, uint16_t* out, long long ldo, const uint16_t* A, int lda, int M, const awq_qweight* w,
-                           int K, int N, int accum);
+                           int K, int N, int accum, bool static_ws);
 int awq_launch_gemm_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, long long kv_row0_off,
                         const uint16_t* A, int lda, int M, const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw,
                         int K, int Nq, int Nkv, const float2* rope128, int pos0);
@@ -775,10 +775,10 @@ int awq_transformer_prefill(awq_transformer* t, int n_tokens, int gen_token) {
             if ((r = awq_launch_attn_prefill(ctx, t->pf_att, t->pf_q, t->s.key_cache + loff, t->s.value_cache + loff, p.n_heads, hs,
                                              kv_mul, M, pos0)))
                 return r;
-            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_att, dim, M, &L.wq_o, dim, dim, 1))) return r;
+            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_att, dim, M, &L.wq_o, dim, dim, 1, false))) return r;
             if ((r = awq_launch_rmsnorm_rows(ctx, t->pf_xb, t->pf_x, L.rms_ffn_weight, dim, M))) return r;
             if ((r = awq_launch_gemm_ffn(ctx, t->pf_hb, t->pf_xb, dim, M, &L.wq_gate, &L.wq_up, dim, hidden))) return r;
-            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_hb, hidden, M, &L.wq_down, hidden, dim, 1))) return r;
+            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_hb, hidden, M, &L.wq_down, hidden, dim, 1, false))) return r;
         }
         if (done + M == n_tokens) {
             // last token: final norm, classifier and the greedy sampler exactly as the decode path does them

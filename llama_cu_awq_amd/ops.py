@@ -217,3 +217,8 @@ def dequant(ctx, out, w, K, N):
 def gemm_q(ctx, out, ldo, a, lda, M, w, K, N, accum=False):
     """Batched form of matmul(QWeight) for M activation rows (prefill); no launcher of this kind exists in the reference."""
     check(lib.awq_gemm_int4(ctx.h, _addr(out), ldo, _addr(a), lda, M, C.byref(w.c), K, N, int(accum)))
+
+
+def gemm_q_static(ctx, out, ldo, a, lda, M, w, K, N, accum=False):
+    """gemm_q() with the split-K workspace in the library's own device array: allocates nothing (for callers under graph capture)."""
+    check(lib.awq_gemm_int4_static(ctx.h, _addr(out), ldo, _addr(a), lda, M, C.byref(w.c), K, N, int(accum)))
