@@ -5,13 +5,16 @@ A step is one token through the whole network (one pass of the hot path).  The d
 random prompt as warm-up and times exactly 256 decode steps; weights are random (no checkpoints offline) with the
 real layout and distributions, resident in HBM before the timed region starts.
 
-Prints ONE JSON line: tokens/s (`value`), the roofline of the dominant kernel (the fused gate/up int4
-matrix-vector product) measured live with HIP events over distinct per-layer weights, and the CPU oracle timed
-on a bounded sample of the same workload.
+Prints ONE JSON line: tokens/s (`value`) of the run the flags ask for; `config1`, the benchmark's own run (16-token
+prompt + 256 decode steps from position 0) whatever the flags were; the roofline of the dominant kernel as the timed
+schedule launches it (RMSNorm-fused gate/up int4 matrix-vector product, timed live with HIP events over the 32
+layers' distinct weights); `config0`, the single 4096 x 4096 product back to back on one stream and dealt over 2 and 4
+plain streams; the 512-token prefill; and the CPU oracle timed on a bounded sample of the same workload.
 """
 import argparse
 import json
 import os
+import subprocess
 import sys
 import time
 
@@ -20,6 +23,16 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # MI355X published HBM3E bandwidth, bytes/s
+
+# Figures that cannot be measured inside this process (hardware counters, profiler durations): read from the
+# rocprofv3 summaries committed under profiles/, each named with its source.
+PROFILED = {
+    # HBM bytes per launch of the norm-fused gate/up kernel at the 7B shape: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
+    "ffn_traffic_bytes": (47063305, "profiles/gemv_int4_ffn_7b_pmc.md"),
+    # rocprofv3 --kernel-trace average durations in the decode run, microseconds
+    "ffn_kernel_us": (11.62, "profiles/decode_7b_fused_kernel_trace.md"),
+    "gemv_4096_kernel_us": (4.19, "profiles/decode_7b_fused_kernel_trace.md"),
+}
 
 
 def qweight_bytes(K, N):
@@ -75,7 +88,6 @@ def main():
     vocab = cfg["vocab_size"]
     kv_dim = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"]
     prompt = synth.prompt_tokens(args.seed, n_prompt, vocab)
-    model.reset(prompt)
     if args.start_pos:
         # KV cache pre-filled with N(0,1) below start_pos (long-context configuration)
         for name in ("key_cache", "value_cache"):
@@ -83,13 +95,34 @@ def main():
             for l in range(cfg["n_layers"]):
                 vals = synth.normal_f16(synth.stream_key(args.seed, name, l), args.start_pos * kv_dim)
                 buf.write(vals, offset_bytes=l * cfg["seq_len"] * kv_dim * 2)
-        model.set_pos(args.start_pos, prompt[0])
-        tok = (np.ctypeslib.as_array(model._tokens))
-        tok[args.start_pos : args.start_pos + n_prompt] = prompt
 
-    def step(i):
-        ctx.sync()  # the reference loop waits for the previous token before launching the next (llama2_q4.cu:713)
-        model.forward(gen_token=(i >= n_prompt - 1), use_graph=use_graph, mode=mode)
+    def run_decode(n_prompt, n_steps, start_pos=0):
+        """Prompt as warm-up, then n_steps timed decode steps with the reference's synchronise-then-launch loop
+        (llama2_q4.cu:713).  Every recorded launch sequence the run will replay is recorded before the clock starts."""
+        toks = synth.prompt_tokens(args.seed, n_prompt, vocab)
+        model.reset(toks)
+        if start_pos:
+            model.set_pos(start_pos, toks[0])
+            np.ctypeslib.as_array(model._tokens)[start_pos : start_pos + n_prompt] = toks
+            for i, tk in enumerate(toks):  # the device mirror of the token list, which the fused schedule reads
+                model.set_pos(start_pos + i, tk)
+            model.set_pos(start_pos, toks[0])
+        if use_graph and mode != A.SCHEDULE_PERSISTENT:
+            model.capture(start_pos + n_prompt + n_steps, mode)
+        for i in range(n_prompt):
+            ctx.sync()
+            model.forward(gen_token=(i >= n_prompt - 1), use_graph=use_graph, mode=mode)
+        ctx.sync()
+        ctx.record(ev0)
+        w0 = time.perf_counter()
+        for i in range(n_steps):
+            ctx.sync()
+            model.forward(gen_token=True, use_graph=use_graph, mode=mode)
+        ctx.record(ev1)
+        ctx.sync()
+        wall = time.perf_counter() - w0
+        first = start_pos + n_prompt
+        return wall, ctx.elapsed_ms(ev0, ev1), [model.token(first + i) for i in range(min(8, n_steps))]
 
     ev0, ev1 = ctx.event(), ctx.event()
     if args.only_kernels:
@@ -103,65 +136,93 @@ def main():
             check(lib.awq_memcpy_d2d_async(ctx.h, dst.ptr, src.ptr, nbytes))
         ctx.sync()
         args.steps, n_prompt, total = 1, 1, 2
-    for i in range(n_prompt):  # warm-up: the prompt
-        step(i)
-    ctx.sync()
-    ctx.record(ev0)
-    w0 = time.perf_counter()
-    for i in range(n_prompt, total):
-        step(i)
-    ctx.record(ev1)
-    ctx.sync()
-    wall = time.perf_counter() - w0
-    gpu_ms = ctx.elapsed_ms(ev0, ev1)
+    wall, gpu_ms, gen = run_decode(n_prompt, args.steps, args.start_pos)
     tok_s = args.steps / wall
-    first = args.start_pos + n_prompt
-    gen = [model.token(first + i) for i in range(min(8, args.steps))]
 
     wbytes = weight_bytes_per_token(cfg)
     avg_kv = 2 * cfg["n_layers"] * kv_dim * 2 * (args.start_pos + n_prompt + (args.steps + 1) / 2.0)
     decode_gbps = (wbytes + avg_kv) * tok_s / 1e9
 
-    # ---- dominant kernel: fused gate/up int4 matvec + SiLU*mul, one launch per layer over that layer's own weights
+    # ---- dominant kernel, as the timed (fused) schedule launches it: RMSNorm folded into the staging of x, gate and up
+    # rows walked together, SiLU(gate) * up in the epilogue; one launch per layer over that layer's own weights (1.5 GB
+    # of distinct matrices at 7B, so the 256 MB memory-side cache cannot serve them), timed with events on the
+    # context's stream.  The plain form (separate RMSNorm, what the reference schedule launches) is timed beside it.
     dim, hid = cfg["dim"], cfg["hidden_dim"]
     layers = [model.layer(l) for l in range(cfg["n_layers"])]
+    xres = model.buffer("x", dim * 2)
     xb = model.buffer("xb", dim * 2)
     hb = model.buffer("hb", hid * 2)
     reps = 8
 
-    def ffn_pass():
+    def timed(fn):
+        fn()
+        ctx.sync()
+        ctx.record(ev0)
+        for _ in range(reps):
+            fn()
+        ctx.record(ev1)
+        ctx.sync()
+        return ctx.elapsed_ms(ev0, ev1) * 1e3 / reps
+
+    def ffn_fused_pass():
+        for L in layers:
+            A.rmsnorm_ffn_matvec_silu(ctx, hb, xres, L["rms_ffn_weight"], L["wq_gate"], L["wq_up"], dim, hid)
+
+    def ffn_plain_pass():
         for L in layers:
             A.ffn_matvec_silu(ctx, hb, xb, L["wq_gate"], L["wq_up"], dim, hid)
 
-    ffn_pass()
-    ctx.sync()
-    ctx.record(ev0)
-    for _ in range(reps):
-        ffn_pass()
-    ctx.record(ev1)
-    ctx.sync()
-    ffn_us = ctx.elapsed_ms(ev0, ev1) * 1e3 / (reps * len(layers))
-    ffn_bytes = 2 * qweight_bytes(dim, hid) + dim * 2 + hid * 2
+    ffn_us = timed(ffn_fused_pass) / len(layers)
+    ffn_plain_us = timed(ffn_plain_pass) / len(layers)
+    ffn_bytes = 2 * qweight_bytes(dim, hid) + dim * 2 + dim * 2 + hid * 2  # weights, x, norm weights, out
     ffn_gbps = ffn_bytes / ffn_us / 1e3
+    ffn_waves = 4 if dim <= 8192 else 16
 
-    # ---- the single 4096x4096-class GEMV (q/k/v/o shapes), rotating over every layer's four matrices
-    resid = model.buffer("x", dim * 2)
-
+    # ---- configuration 0: the single dim x dim product (q/k/v/o shapes), rotating over every layer's four matrices
     def gemv_pass():
         for L in layers:
             for n in ("wq_q", "wq_k", "wq_v", "wq_o"):
-                A.matmul_q(ctx, resid, xb, L[n], dim, dim)
+                A.matmul_q(ctx, hb, xb, L[n], dim, dim)
 
-    gemv_pass()
-    ctx.sync()
-    ctx.record(ev0)
-    for _ in range(reps):
-        gemv_pass()
-    ctx.record(ev1)
-    ctx.sync()
-    gemv_us = ctx.elapsed_ms(ev0, ev1) * 1e3 / (reps * len(layers) * 4)
+    gemv_us = timed(gemv_pass) / (len(layers) * 4)
     gemv_bytes = qweight_bytes(dim, dim) + 4 * dim
     gemv_gbps = gemv_bytes / gemv_us / 1e3
+    config0 = {
+        "shape": [dim, dim],
+        "bytes_per_product": gemv_bytes,
+        "one_stream_back_to_back": {"us_per_product": round(gemv_us, 3), "gbps": round(gemv_gbps, 1), "frac": round(gemv_gbps * 1e9 / HBM_PEAK, 4)},
+    }
+    if (dim, hid) == (4096, 11008):
+        us, src = PROFILED["gemv_4096_kernel_us"]
+        config0["rocprof_kernel_duration"] = {"us_per_product": us, "gbps": round(gemv_bytes / us / 1e3, 1), "frac": round(gemv_bytes / us / 1e3 / 8000.0, 4), "source": src}
+    # the same product through the C-ABI from one host thread per stream: 1, 2 and 4 plain streams over 64 distinct
+    # matrices (558 MB), so that the fixed cost of a dependent launch overlaps the streaming of the other streams
+    tool = os.path.join(ROOT, "llama_cu_awq_amd", "bin", "gemv_bench")
+    if os.path.exists(tool) and not args.only_kernels:
+        try:
+            res = subprocess.run([tool, str(dim), str(dim), "64", "8"], capture_output=True, text=True, timeout=120)
+            if res.returncode == 0:
+                config0["independent_streams"] = json.loads(res.stdout.strip().splitlines()[-1])
+            else:
+                config0["independent_streams"] = {"error": res.stderr.strip()[-200:]}
+        except Exception as e:  # the tool is a side measurement; the benchmark line does not depend on it
+            config0["independent_streams"] = {"error": str(e)[-200:]}
+
+    # ---- configuration 1 (the benchmark's own run), whatever --steps / --warmup were
+    config1 = None
+    if args.config == "7b" and not args.only_kernels:
+        if (n_prompt, args.steps, args.start_pos) == (16, 256, 0):
+            c_wall, c_gpu_ms, c_gen = wall, gpu_ms, gen
+        else:
+            c_wall, c_gpu_ms, c_gen = run_decode(16, 256, 0)
+        config1 = {
+            "workload": "16-token prompt then 256 decode steps from position 0",
+            "tok_per_s": round(256 / c_wall, 2),
+            "ms_per_step": round(c_wall * 1e3 / 256, 4),
+            "gpu_ms_per_step": round(c_gpu_ms / 256, 4),
+            "frac_of_weight_roofline": round(256 / c_wall / (HBM_PEAK / weight_bytes_per_token(cfg)), 4),
+            "first_tokens": c_gen,
+        }
 
     # ---- prefill (7B shape, M prompt tokens in one batched pass on the matrix cores)
     prefill = None
@@ -231,15 +292,21 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_int4_kernel<8 waves, 1 row pair, 2 passes in flight, FFN> (fused gate/up + SiLU*mul), K=%d N=%d" % (dim, hid),
+            "kernel": "gemv_int4_kernel<W=%d waves, R=1 gate/up row pair per wave, D=2 passes in flight, KIND_FFN, NORM=true, ROPE=false> "
+            "(RMSNorm while staging x, SiLU(gate)*up epilogue; the launch of the fused schedule), K=%d N=%d" % (ffn_waves, dim, hid),
             "achieved": round(ffn_gbps, 1),
             "peak": HBM_PEAK / 1e9,
             "unit": "GB/s",
             "frac": round(ffn_gbps * 1e9 / HBM_PEAK, 4),
-            # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE (7B shape; profiles/gemv_int4_ffn_7b_pmc.md)
-            "traffic": 47063305 if (dim, hid) == (4096, 11008) else None,
+            # HBM bytes per launch cannot be counted from inside the run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this
+            # kernel at the 7B shape, from the committed summary
+            "traffic": PROFILED["ffn_traffic_bytes"][0] if (dim, hid) == (4096, 11008) else None,
+            "traffic_source": PROFILED["ffn_traffic_bytes"][1] if (dim, hid) == (4096, 11008) else None,
             "bytes_per_launch": ffn_bytes,
             "us_per_launch": round(ffn_us, 3),
+            "rocprof_us_per_launch": PROFILED["ffn_kernel_us"][0] if (dim, hid) == (4096, 11008) else None,
+            "rocprof_source": PROFILED["ffn_kernel_us"][1] if (dim, hid) == (4096, 11008) else None,
+            "plain_form_us_per_launch": round(ffn_plain_us, 3),
         },
         "cpu_baseline": cpu,
         "prefill": prefill,
@@ -251,7 +318,8 @@ def main():
             "frac_of_weight_roofline": round(tok_s / (HBM_PEAK / wbytes), 4),
             "first_tokens": gen,
         },
-        "gemv_int4_%dx%d" % (dim, dim): {"us_per_launch": round(gemv_us, 3), "bytes": gemv_bytes, "gbps": round(gemv_gbps, 1), "frac": round(gemv_gbps * 1e9 / HBM_PEAK, 4)},
+        "config0": config0,
+        "config1": config1,
     }
     print(json.dumps(out), flush=True)
     model.close()

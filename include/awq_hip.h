@@ -113,6 +113,12 @@ int awq_qkv_matvec(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* val
 int awq_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w,
                         const awq_qweight* up_w, int K, int N);
 
+/* rmsnorm() followed by ffn_matvec_silu() (llama2_q4.cu:496-498) as ONE launch, the form the fused schedule issues:
+ * out = half(silu(Wgate xn) * (Wup xn)) with xn = half(x * (rsqrt(mean(x^2) + 1e-5) * norm_weight)) formed while x
+ * is staged; xn never travels through memory.  Same rounding points as the two separate calls. */
+int awq_rmsnorm_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* norm_weight,
+                                const awq_qweight* gate_w, const awq_qweight* up_w, int K, int N);
+
 /* RoPERotation(), llama2_q4.cu:406-408: rotate-half RoPE, pairs (i, i+head/2), in place on q (all heads)
  * and on the K row at k + loff + (*pos)*num_kv_heads*head_size (first num_kv_heads heads). */
 int awq_rope(awq_ctx* ctx, uint16_t* q, uint16_t* k, int num_heads, int num_kv_heads, int head_size, const int* pos,
@@ -202,6 +208,12 @@ int awq_transformer_set_pos(awq_transformer* t, int pos, int token);
 #define AWQ_SCHEDULE_FUSED 1
 #define AWQ_SCHEDULE_PERSISTENT 2
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode);
+
+/* Record and instantiate ahead of time the launch sequences that awq_transformer_forward(use_graph != 0) replays for
+ * positions below max_positions (one per sequence-length bin, llama2_q4.cu:553-575, where the reference records a bin
+ * on its first visit, inside the decode loop).  Executes nothing; the run state is untouched.  mode: REFERENCE or
+ * FUSED. */
+int awq_transformer_capture(awq_transformer* t, int mode, int max_positions);
 
 /* run_llama_network() alone (llama2_q4.cu:430-538): the token's logits without any sampler, for callers that sample
  * on their own (the non-greedy branch of sample(), sampler.h:85-115).  mode: REFERENCE or FUSED; launched eagerly. */

@@ -17,6 +17,7 @@ from .ops import (  # noqa: F401
     matmul_q,
     qkv_matvec,
     rmsnorm,
+    rmsnorm_ffn_matvec_silu,
     sample_top_p,
     softmax_logits,
 )

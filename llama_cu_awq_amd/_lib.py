@@ -64,6 +64,7 @@ PROTOTYPES = {
     "awq_matvec_int4": [_vp, _vp, _vp, _pq, _i, _i, _i, _i, _i, _vp],
     "awq_qkv_matvec": [_vp, _vp, _vp, _vp, _vp, _pq, _pq, _pq, _i, _i, _i, _vp],
     "awq_ffn_matvec_silu": [_vp, _vp, _vp, _pq, _pq, _i, _i],
+    "awq_rmsnorm_ffn_matvec_silu": [_vp, _vp, _vp, _vp, _pq, _pq, _i, _i],
     "awq_rope": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _f],
     "awq_attention": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "awq_matvec_f16": [_vp, _vp, _vp, _vp, _i, _i],
@@ -79,6 +80,7 @@ PROTOTYPES = {
     "awq_transformer_reset": [_vp, C.POINTER(C.c_int), _i],
     "awq_transformer_set_pos": [_vp, _i, _i],
     "awq_transformer_forward": [_vp, _i, _i, _i],
+    "awq_transformer_capture": [_vp, _i, _i],
     "awq_gemm_int4": [_vp, _vp, _i, _vp, _i, _i, _pq, _i, _i, _i],
     "awq_gemm_int4_static": [_vp, _vp, _i, _vp, _i, _i, _pq, _i, _i, _i],
     "awq_transformer_prefill": [_vp, _i, _i],

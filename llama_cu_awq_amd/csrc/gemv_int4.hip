@@ -456,6 +456,14 @@ int awq_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const aw
     return awq_launch_ffn(ctx, out, x, gate_w, up_w, K, N, nullptr, nullptr);
 }
 
+int awq_rmsnorm_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* norm_weight,
+                                const awq_qweight* gate_w, const awq_qweight* up_w, int K, int N) {
+    if (int r = awq_bind(ctx)) return r;
+    if (int r = check_shape(K, N)) return r;
+    AWQ_REQUIRE(out && x && norm_weight && qw_ok(gate_w) && qw_ok(up_w), AWQ_ERR_ARG, "null pointer");
+    return awq_launch_ffn(ctx, out, x, gate_w, up_w, K, N, norm_weight, nullptr);
+}
+
 int awq_dequant(awq_ctx* ctx, uint16_t* out, const awq_qweight* w, int K, int N) {
     if (int r = awq_bind(ctx)) return r;
     if (K <= 0 || N <= 0 || (K & 7) || (N & 7)) {

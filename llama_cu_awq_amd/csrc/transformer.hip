@@ -516,6 +516,47 @@ int network(awq_transformer* t, int seq_len_bin, int mode) {
     return mode == AWQ_SCHEDULE_FUSED ? network_fused(t, seq_len_bin) : network_reference(t, seq_len_bin);
 }
 
+// llama2_q4.cu:553-558: sequence-length bins 128, 256, ..., the last one being the model's seq_len.  Returns the
+// index of the bin that a pass over seq_len positions replays and stores the bin's launch size.
+int graph_bin(const awq_config& cfg, int seq_len, int* seq_len_bin_out) {
+    int graph_index;
+    int seq_len_bin = 128;
+    for (graph_index = 0; graph_index < kMaxGraphs - 1; seq_len_bin *= 2, graph_index++)
+        if (seq_len <= seq_len_bin) break;
+    if (seq_len > seq_len_bin || graph_index == kMaxGraphs - 1 || seq_len_bin > cfg.seq_len) seq_len_bin = cfg.seq_len;
+    *seq_len_bin_out = seq_len_bin;
+    return graph_index;
+}
+
+// Record and instantiate the launch sequence (network + greedy sampler) of one bin, unless that is done already.
+// Recording executes nothing and leaves the run state untouched.
+int ensure_captured(awq_transformer* t, int mode, int graph_index, int seq_len_bin) {
+    if (t->captured[mode][graph_index]) return AWQ_OK;
+    awq_ctx* ctx = t->ctx;
+    hipGraph_t graph = nullptr;
+    AWQ_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+    int r = network(t, seq_len_bin, mode);
+    if (r == AWQ_OK)
+        r = awq_launch_argmax(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, 1, t->tokens_dev);
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (r) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return r;
+    }
+    if (e != hipSuccess) {
+        awq_set_error("hipStreamEndCapture failed: %s", hipGetErrorString(e));
+        return AWQ_ERR_HIP;
+    }
+    e = hipGraphInstantiate(&t->graphs[mode][graph_index], graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) {
+        awq_set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
+        return AWQ_ERR_HIP;
+    }
+    t->captured[mode][graph_index] = true;
+    return AWQ_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -860,6 +901,25 @@ int awq_transformer_sample(awq_transformer* t, awq_sampler* sampler, int gen_tok
     return AWQ_OK;
 }
 
+int awq_transformer_capture(awq_transformer* t, int mode, int max_positions) {
+    AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
+    AWQ_REQUIRE(mode == AWQ_SCHEDULE_REFERENCE || mode == AWQ_SCHEDULE_FUSED, AWQ_ERR_ARG,
+                "only the reference and the fused schedule replay recorded sequences");
+    AWQ_REQUIRE(max_positions >= 1 && max_positions <= t->cfg.seq_len, AWQ_ERR_ARG, "max_positions out of range");
+    if (int r = awq_bind(t->ctx)) return r;
+    int last = -1;
+    for (int seq_len = 1; seq_len <= max_positions; seq_len++) {
+        int seq_len_bin;
+        const int graph_index = graph_bin(t->cfg, seq_len, &seq_len_bin);
+        if (graph_index != last) {
+            if (int r = ensure_captured(t, mode, graph_index, seq_len_bin)) return r;
+            last = graph_index;
+        }
+        seq_len = (seq_len_bin < max_positions ? seq_len_bin : max_positions);  // jump to the end of this bin
+    }
+    return AWQ_OK;
+}
+
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode) {
     AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
     AWQ_REQUIRE(mode == AWQ_SCHEDULE_REFERENCE || mode == AWQ_SCHEDULE_FUSED || mode == AWQ_SCHEDULE_PERSISTENT, AWQ_ERR_ARG,
@@ -889,31 +949,9 @@ int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, in
     AWQ_REQUIRE(seq_len <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
     int r;
     if (use_graph) {
-        // llama2_q4.cu:553-558: bins 128, 256, ..., last bin = seq_len of the model
-        int graph_index;
-        int seq_len_bin = 128;
-        for (graph_index = 0; graph_index < kMaxGraphs - 1; seq_len_bin *= 2, graph_index++)
-            if (seq_len <= seq_len_bin) break;
-        if (seq_len > seq_len_bin || graph_index == kMaxGraphs - 1 || seq_len_bin > t->cfg.seq_len) seq_len_bin = t->cfg.seq_len;
-        if (!t->captured[mode][graph_index]) {
-            hipGraph_t graph = nullptr;
-            AWQ_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
-            r = network(t, seq_len_bin, mode);
-            if (r == AWQ_OK)
-                r = awq_launch_argmax(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, 1, t->tokens_dev);
-            hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
-            if (r) {
-                if (graph) (void)hipGraphDestroy(graph);
-                return r;
-            }
-            if (e != hipSuccess) {
-                awq_set_error("hipStreamEndCapture failed: %s", hipGetErrorString(e));
-                return AWQ_ERR_HIP;
-            }
-            AWQ_HIP_TRY(hipGraphInstantiate(&t->graphs[mode][graph_index], graph, nullptr, nullptr, 0));
-            AWQ_HIP_TRY(hipGraphDestroy(graph));
-            t->captured[mode][graph_index] = true;
-        }
+        int seq_len_bin;
+        const int graph_index = graph_bin(t->cfg, seq_len, &seq_len_bin);
+        if ((r = ensure_captured(t, mode, graph_index, seq_len_bin))) return r;
         // The recorded sampler always writes its token; while the prompt is being consumed the next prompt
         // token must survive, so those steps run eagerly below.
         if (gen_token) {

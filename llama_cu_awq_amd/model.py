@@ -70,6 +70,10 @@ class Transformer:
     def forward(self, gen_token=True, use_graph=False, mode=SCHEDULE_FUSED):
         check(lib.awq_transformer_forward(self.h, int(gen_token), int(use_graph), mode))
 
+    def capture(self, max_positions, mode=SCHEDULE_FUSED):
+        """Record the launch sequences of every sequence-length bin below max_positions ahead of time."""
+        check(lib.awq_transformer_capture(self.h, mode, max_positions))
+
     def forward_logits(self, use_graph=False, mode=SCHEDULE_FUSED):
         """run_llama_network() alone: this position's logits, no sampler."""
         check(lib.awq_transformer_forward_logits(self.h, int(use_graph), mode))

@@ -161,6 +161,11 @@ def ffn_matvec_silu(ctx, xout, x, gate_w, up_w, inpSize, opSize):
     check(lib.awq_ffn_matvec_silu(ctx.h, _addr(xout), _addr(x), C.byref(gate_w.c), C.byref(up_w.c), inpSize, opSize))
 
 
+def rmsnorm_ffn_matvec_silu(ctx, xout, x, norm_weight, gate_w, up_w, inpSize, opSize):
+    """rmsnorm() + ffn_matvec_silu() (llama2_q4.cu:496-498) in one launch: what the fused schedule issues."""
+    check(lib.awq_rmsnorm_ffn_matvec_silu(ctx.h, _addr(xout), _addr(x), _addr(norm_weight), C.byref(gate_w.c), C.byref(up_w.c), inpSize, opSize))
+
+
 def RoPERotation(ctx, q, k, num_heads, num_kv_heads, head_size, pPos, loff, rope_theta):
     """RoPERotation(), llama2_q4.cu:406-408."""
     check(lib.awq_rope(ctx.h, _addr(q), _addr(k), num_heads, num_kv_heads, head_size, _addr(pPos), loff, rope_theta))

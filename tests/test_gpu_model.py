@@ -76,6 +76,96 @@ def test_greedy_decode_matches_oracle(pair, mode, graph):
     assert worst <= 1e-2, worst
 
 
+def test_capture_ahead_of_time_changes_nothing(ctx):
+    """Recording every bin up front (seq_len 300: bins 128, 256 and the model's own length) leaves the run state alone
+    and gives the tokens of a run that records on first visit; the bins are crossed inside the run."""
+    cfg = dict(dim=256, hidden_dim=768, n_layers=2, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=300, rope_theta=10000.0)
+    img = synth.make_model_image(cfg, seed=8, scale_mult=0.25)
+    prompt = synth.prompt_tokens(8, 4, cfg["vocab_size"])
+    o = oracle.Model(img)
+    want, _, _ = o.generate(prompt, 299, ignore_eos=True)
+    o.close()
+    runs = []
+    for ahead in (False, True):
+        t = A.Transformer(ctx, image=img)
+        t.reset(prompt)
+        if ahead:
+            t.forward(False, True, A.SCHEDULE_FUSED)  # something in flight and a position other than 0
+            t.capture(cfg["seq_len"], A.SCHEDULE_FUSED)
+            t.capture(cfg["seq_len"], A.SCHEDULE_REFERENCE)
+            ctx.sync()
+            assert t.pos == 1
+            t.reset(prompt)
+        toks, pos = t.generate(prompt, 299, ignore_eos=True, use_graph=True, mode=A.SCHEDULE_FUSED)
+        assert pos == 299
+        runs.append(toks)
+        with pytest.raises(A.AwqError):
+            t.capture(cfg["seq_len"] + 1)
+        t.close()
+    assert runs[0] == runs[1]
+    agree = next((i for i in range(300) if runs[0][i] != want[i]), 300)
+    assert agree > 4 + 32, agree  # greedy tokens as the oracle's well past the benchmark's 32 steps
+
+
+def test_context_and_model_handed_between_host_threads():
+    """The reference allocates on one short-lived thread, issues every launch from another and tears down from the
+    main thread (llama2_q4.cu:613-623, 685, 776-783).  Same hand-off through the C-ABI: context + model created on
+    thread A (which exits), decode loop on thread B under graph replay and eagerly, prefill on thread C, free on
+    thread D; the tokens are the oracle's."""
+    import threading
+
+    cfg = dict(SMALL, hidden_dim=2816)  # multiples of 128, as the batched prefill needs
+    img = synth.make_model_image(cfg, seed=11, scale_mult=0.25)
+    prompt = synth.prompt_tokens(11, 6, cfg["vocab_size"])
+    o = oracle.Model(img)
+    want, _, _ = o.generate(prompt, 40, ignore_eos=True)
+    o.close()
+    box, errors = {}, []
+
+    def on_thread(fn):
+        def run():
+            try:
+                fn()
+            except BaseException as e:  # surfaced in the main thread below
+                errors.append(e)
+
+        th = threading.Thread(target=run)
+        th.start()
+        th.join()
+        assert not errors, errors
+
+    def create():
+        box["ctx"] = A.Context(0)
+        box["t"] = A.Transformer(box["ctx"], image=img)
+
+    def decode(graph):
+        def fn():
+            box[graph] = box["t"].generate(prompt, 40, ignore_eos=True, use_graph=graph, mode=A.SCHEDULE_FUSED)[0]
+
+        return fn
+
+    def prefill():
+        t = box["t"]
+        t.reset(prompt)
+        t.prefill(len(prompt), gen_token=True)
+        box["ctx"].sync()
+        box["next"] = t.token(len(prompt))
+
+    def destroy():
+        box["t"].close()
+        box["ctx"].close()
+
+    on_thread(create)
+    on_thread(decode(True))
+    on_thread(decode(False))
+    on_thread(prefill)
+    on_thread(destroy)
+    agree = next((i for i in range(41) if box[True][i] != want[i]), 41)
+    assert agree > 6 + 32, agree
+    assert box[True] == box[False]
+    assert box["next"] == want[len(prompt)]
+
+
 def test_eos_stops_generation(pair):
     """The loop breaks when token 2 is read back (llama2_q4.cu:730)."""
     cfg, t, o = pair

@@ -139,6 +139,33 @@ def test_qkv_matvec(ctx, K, N):
     assert rel_l2(f16(kgot[loff + pos * N : loff + (pos + 1) * N]), truth) <= 1e-3
 
 
+@pytest.mark.parametrize("K,N", [(4096, 11008), (5120, 13824), (6656, 17920), (256, 72), (1024, 4480)])
+def test_rmsnorm_ffn_matvec_silu_equals_the_two_calls(ctx, K, N):
+    """The one-launch form of rmsnorm + ffn_matvec_silu (what the fused schedule runs) against the oracle's two steps:
+    the normalised vector must be the same fp16 values, so the outputs agree as closely as the plain kernel's do."""
+    gate = _case(K, N, 23)[:3]
+    up = _case(K, N, 24)[:3]
+    x = (_case(K, N, 25)[3].astype(np.float32) * 3.0).astype(np.float16)  # a residual stream, not a normalised vector
+    nw = synth.normal_f16(synth.stream_key(1, "nw", K), K, 1.0, 0.02)
+    dout = ctx.zeros(N * 2)
+    A.rmsnorm_ffn_matvec_silu(ctx, dout, ctx.upload(x), ctx.upload(nw), A.QWeight.upload(ctx, *gate), A.QWeight.upload(ctx, *up), K, N)
+    got = f16(dout.download(np.uint16))
+    xn = oracle.rmsnorm(x, nw)
+    want = np.zeros(N, dtype=np.uint16)
+    oracle.ffn_matvec_silu(want, xn, gate, up, K, N)
+    xd = xn.astype(np.float64)
+    g = synth.dequantize(*gate, K) @ xd
+    u = synth.dequantize(*up, K) @ xd
+    assert rel_l2(got, g / (1.0 + np.exp(-g)) * u) <= 1e-3
+    assert rel_l2(got, f16(want)) <= 3e-4
+    # and against the library's own two launches
+    dxn, d2 = ctx.zeros(K * 2), ctx.zeros(N * 2)
+    A.rmsnorm(ctx, dxn, ctx.upload(x), ctx.upload(nw), K)
+    assert ulp_diff_f16(f16(dxn.download(np.uint16)), xn).max() <= 1  # the sum of squares is added in another order
+    A.ffn_matvec_silu(ctx, d2, dxn, A.QWeight.upload(ctx, *gate), A.QWeight.upload(ctx, *up), K, N)
+    assert_close_f16(got, f16(d2.download(np.uint16)), ulps=2)
+
+
 @pytest.mark.parametrize("K,N", [(4096, 11008), (5120, 13824), (6656, 1792), (256, 72)])
 def test_ffn_matvec_silu(ctx, K, N):
     gate = _case(K, N, 20)[:3]
