@@ -28,10 +28,10 @@ HBM_PEAK = 8.0e12  # MI355X published HBM3E bandwidth, bytes/s
 # rocprofv3 summaries committed under profiles/, each named with its source.
 PROFILED = {
     # HBM bytes per launch of the norm-fused gate/up kernel at the 7B shape: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
-    "ffn_traffic_bytes": (47063305, "profiles/gemv_int4_ffn_7b_pmc.md"),
+    "ffn_traffic_bytes": (47561728, "profiles/gemv_int4_ffn_7b_pmc.md"),
     # rocprofv3 --kernel-trace average durations in the decode run, microseconds
-    "ffn_kernel_us": (11.62, "profiles/decode_7b_fused_kernel_trace.md"),
-    "gemv_4096_kernel_us": (4.19, "profiles/decode_7b_fused_kernel_trace.md"),
+    "ffn_kernel_us": (11.11, "profiles/decode_7b_fused_kernel_trace.md"),
+    "gemv_4096_kernel_us": (4.14, "profiles/decode_7b_fused_kernel_trace.md"),
 }
 
 
@@ -172,8 +172,14 @@ def main():
         for L in layers:
             A.ffn_matvec_silu(ctx, hb, xb, L["wq_gate"], L["wq_up"], dim, hid)
 
-    ffn_us = timed(ffn_fused_pass) / len(layers)
+    ffn_loop_us = timed(ffn_fused_pass) / len(layers)
     ffn_plain_us = timed(ffn_plain_pass) / len(layers)
+    # ... and where it actually runs: every kernel of the fused schedule timed in place (eager passes at the middle
+    # position of the timed run, each kernel launched with an event pair stamped with its own start and end)
+    mid = args.start_pos + n_prompt + args.steps // 2
+    model.set_pos(min(mid, cfg["seq_len"] - 1), prompt[0])
+    in_place = model.time_launches(passes=4)
+    ffn_us = in_place["gate_up"]["us"]
     ffn_bytes = 2 * qweight_bytes(dim, hid) + dim * 2 + dim * 2 + hid * 2  # weights, x, norm weights, out
     ffn_gbps = ffn_bytes / ffn_us / 1e3
     ffn_waves = 4 if dim <= 8192 else 16
@@ -304,6 +310,8 @@ def main():
             "traffic_source": PROFILED["ffn_traffic_bytes"][1] if (dim, hid) == (4096, 11008) else None,
             "bytes_per_launch": ffn_bytes,
             "us_per_launch": round(ffn_us, 3),
+            "how_timed": "start/stop HIP events attached to each of the %d gate/up launches (kernel start to kernel end) in 4 eager passes of the fused schedule at position %d, on the context's stream" % (cfg["n_layers"], mid),
+            "isolated_loop_us_per_launch": round(ffn_loop_us, 3),
             "rocprof_us_per_launch": PROFILED["ffn_kernel_us"][0] if (dim, hid) == (4096, 11008) else None,
             "rocprof_source": PROFILED["ffn_kernel_us"][1] if (dim, hid) == (4096, 11008) else None,
             "plain_form_us_per_launch": round(ffn_plain_us, 3),
@@ -318,6 +326,7 @@ def main():
             "frac_of_weight_roofline": round(tok_s / (HBM_PEAK / wbytes), 4),
             "first_tokens": gen,
         },
+        "launches_in_place_us": {k: v["us"] for k, v in in_place.items()},
         "config0": config0,
         "config1": config1,
     }

@@ -215,6 +215,25 @@ int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, in
  * FUSED. */
 int awq_transformer_capture(awq_transformer* t, int mode, int max_positions);
 
+/* Per-launch GPU time of the fused schedule measured in place (the reference's DUMP_PER_TOKEN_TIMINGS switch,
+ * llama2_q4.cu:32, 545-600, times whole tokens; this times each launch of one).  Runs the network of the CURRENT
+ * position `passes` times eagerly (after one untimed run), every kernel launched with an event pair that the runtime
+ * stamps with the kernel's own start and end, and returns, per launch kind, the mean kernel duration in microseconds
+ * and the number of kernels averaged: AWQ_LAUNCH_EMBED, _QKV (RMSNorm + q/k/v products + RoPE), _ATTENTION (each of
+ * its kernels on its own), _OPROJ, _GATE_UP (RMSNorm + gate/up products + SiLU), _DOWN, _CLASSIFIER (RMSNorm + fp16
+ * product).  The gaps between dependent kernels are not part of these figures.  The position is not advanced: the pass rewrites the KV-cache
+ * rows of the current position and the logits with the values a forward call would write.  Both arrays hold
+ * AWQ_LAUNCH_KINDS entries. */
+#define AWQ_LAUNCH_EMBED 0
+#define AWQ_LAUNCH_QKV 1
+#define AWQ_LAUNCH_ATTENTION 2
+#define AWQ_LAUNCH_OPROJ 3
+#define AWQ_LAUNCH_GATE_UP 4
+#define AWQ_LAUNCH_DOWN 5
+#define AWQ_LAUNCH_CLASSIFIER 6
+#define AWQ_LAUNCH_KINDS 7
+int awq_transformer_time_launches(awq_transformer* t, int passes, float* us_by_kind, int* launches_by_kind);
+
 /* run_llama_network() alone (llama2_q4.cu:430-538): the token's logits without any sampler, for callers that sample
  * on their own (the non-greedy branch of sample(), sampler.h:85-115).  mode: REFERENCE or FUSED; launched eagerly. */
 int awq_transformer_forward_logits(awq_transformer* t, int use_graph, int mode);

@@ -81,6 +81,7 @@ PROTOTYPES = {
     "awq_transformer_set_pos": [_vp, _i, _i],
     "awq_transformer_forward": [_vp, _i, _i, _i],
     "awq_transformer_capture": [_vp, _i, _i],
+    "awq_transformer_time_launches": [_vp, _i, C.POINTER(C.c_float), C.POINTER(C.c_int)],
     "awq_gemm_int4": [_vp, _vp, _i, _vp, _i, _i, _pq, _i, _i, _i],
     "awq_gemm_int4_static": [_vp, _vp, _i, _vp, _i, _i, _pq, _i, _i, _i],
     "awq_transformer_prefill": [_vp, _i, _i],

@@ -2,16 +2,29 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
+
+#include <vector>
 
 #include "../../include/awq_hip.h"
 
 // ---------------------------------------------------------------- host side
+// While a context's `probe` is set, every kernel launched through awq_launch() carries an event pair that the
+// runtime stamps with the kernel's own start and end (the launch-with-events form of the HIP extension API), tagged
+// with the kind of schedule step that is current.
+struct awq_launch_probe {
+    std::vector<hipEvent_t> events;  // start, stop, start, stop, ...
+    std::vector<int> kinds;          // one per pair
+    int kind = 0;
+};
+
 struct awq_ctx {
     int device;
     hipStream_t stream;
     bool owns_stream;
+    awq_launch_probe* probe;  // null outside awq_transformer_time_launches
     // Workspace of the prefill GEMM's split-K form (allocated on first use): fp32 partial tiles and per-tile arrival
     // counters (self-resetting).
     float* gemm_part;
@@ -58,6 +71,23 @@ static inline int awq_check_launch(const char* what) {
         return AWQ_ERR_HIP;
     }
     return AWQ_OK;
+}
+
+// Launch on the context's stream; with a probe set, through the extension launch that time-stamps the kernel itself.
+template <typename... Args, typename F = void (*)(Args...)>
+static inline void awq_launch(awq_ctx* ctx, F kernel, dim3 grid, dim3 block, size_t lds, Args... args) {
+    if (ctx->probe) {
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+            hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, ctx->stream, e0, e1, 0, args...);
+            ctx->probe->events.push_back(e0);
+            ctx->probe->events.push_back(e1);
+            ctx->probe->kinds.push_back(ctx->probe->kind);
+            return;
+        }
+        if (e0) (void)hipEventDestroy(e0);
+    }
+    hipLaunchKernelGGL(kernel, grid, block, lds, ctx->stream, args...);
 }
 
 static inline int div_up(int a, int b) { return (a + b - 1) / b; }

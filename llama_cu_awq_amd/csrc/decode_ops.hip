@@ -440,17 +440,17 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
     if (max_seq_len <= kAttnFusedMaxSeq) {
         const size_t lds = (size_t)attention_head_lds_floats(max_seq_len, head_size, 16) * sizeof(float);
         // two workgroups per head (halves of the value dimensions): +0.4 .. 0.7 % tokens/s at 7B; four: no better
-        hipLaunchKernelGGL((attn_fused_kernel<LP, 2>), dim3((num_heads + 7) & ~7, 2), dim3(1024), lds, ctx->stream, output, att, q,
+        awq_launch(ctx, attn_fused_kernel<LP, 2>, dim3((num_heads + 7) & ~7, 2), dim3(1024), lds, output, att, q,
                            key_cache, value_cache, num_heads, head_size, kv_mul, row_stride, alpha, pos, max_seq_len);
         return awq_check_launch("attn_fused");
     }
-    hipLaunchKernelGGL((attn_scores_kernel<LP>), dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, ctx->stream, att, q,
+    awq_launch(ctx, attn_scores_kernel<LP>, dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, att, q,
                        key_cache, head_size, kv_mul, row_stride, alpha, pos);
     if (int r = awq_check_launch("attn_scores")) return r;
     // 16 dimensions (2 lanes x 16 bytes of a row) per workgroup measured best (32: -2.5 %, 8: -4 %, 64: -12 % tokens/s
     // at the 13B shape, 1.6 K context); the head count is padded to a multiple of 8 so that the slices of a head
     // (ids h, h + padded heads, ...) share an XCD and the cache lines they split between them
-    hipLaunchKernelGGL((attn_pv_sliced_kernel<2, 4>), dim3((num_heads + 7) & ~7, LP / 2), dim3(1024), 0, ctx->stream, output, att,
+    awq_launch(ctx, attn_pv_sliced_kernel<2, 4>, dim3((num_heads + 7) & ~7, LP / 2), dim3(1024), 0, output, att,
                        value_cache, num_heads, head_size, kv_mul, row_stride, pos);
     return awq_check_launch("attn_pv_sliced");
 }
@@ -460,7 +460,7 @@ int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const ui
 // Internal: greedy sampler that also records the token in a device-side mirror of the token list.
 int awq_launch_argmax(awq_ctx* ctx, const uint16_t* logits, int size, int* tokens, volatile int* pos_host, int* pos_dev,
                       int write_token, int* tokens_mirror) {
-    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, ctx->stream, logits, size, tokens, pos_host, pos_dev, write_token,
+    awq_launch(ctx, argmax_kernel, dim3(1), dim3(1024), 0, logits, size, tokens, pos_host, pos_dev, write_token,
                        tokens_mirror);
     return awq_check_launch("argmax");
 }
@@ -472,9 +472,9 @@ int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const 
     const dim3 grid(div_up(d, 4 * R));
     const size_t lds = (size_t)n * 2;
     if (norm_w)
-        hipLaunchKernelGGL((gemv_f16_kernel<R, true>), grid, dim3(256), lds, ctx->stream, out, x, w, n, d, norm_w, norm_out);
+        awq_launch(ctx, gemv_f16_kernel<R, true>, grid, dim3(256), lds, out, x, w, n, d, norm_w, norm_out);
     else
-        hipLaunchKernelGGL((gemv_f16_kernel<R, false>), grid, dim3(256), lds, ctx->stream, out, x, w, n, d, norm_w, norm_out);
+        awq_launch(ctx, gemv_f16_kernel<R, false>, grid, dim3(256), lds, out, x, w, n, d, norm_w, norm_out);
     return awq_check_launch("gemv_f16");
 }
 
@@ -484,7 +484,7 @@ int awq_embed(awq_ctx* ctx, uint16_t* x, const uint16_t* table, int dim, const i
     if (int r = awq_bind(ctx)) return r;
     AWQ_REQUIRE(x && table && tokens && pos, AWQ_ERR_ARG, "null pointer");
     AWQ_REQUIRE(dim > 0 && (dim & 7) == 0, AWQ_ERR_SHAPE, "dim must be a positive multiple of 8");
-    hipLaunchKernelGGL(embed_kernel, dim3(div_up(dim >> 3, 256)), dim3(256), 0, ctx->stream, x, table, dim, tokens, pos);
+    awq_launch(ctx, embed_kernel, dim3(div_up(dim >> 3, 256)), dim3(256), 0, x, table, dim, tokens, pos);
     return awq_check_launch("embed");
 }
 
@@ -492,7 +492,7 @@ int awq_rmsnorm(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const uint16_t* we
     if (int r = awq_bind(ctx)) return r;
     AWQ_REQUIRE(o && x && weight, AWQ_ERR_ARG, "null pointer");
     AWQ_REQUIRE(size > 0, AWQ_ERR_SHAPE, "size must be positive");
-    hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(1024), 0, ctx->stream, o, x, weight, size);
+    awq_launch(ctx, rmsnorm_kernel, dim3(1), dim3(1024), 0, o, x, weight, size);
     return awq_check_launch("rmsnorm");
 }
 
@@ -503,7 +503,7 @@ int awq_rope(awq_ctx* ctx, uint16_t* q, uint16_t* k, int num_heads, int num_kv_h
     AWQ_REQUIRE(num_heads > 0 && num_kv_heads >= 0 && num_kv_heads <= num_heads, AWQ_ERR_SHAPE, "bad head counts");
     AWQ_REQUIRE(head_size >= 2 && (head_size & 1) == 0 && head_size <= 2048, AWQ_ERR_SHAPE, "head_size must be even, <= 2048");
     AWQ_REQUIRE(loff >= 0, AWQ_ERR_ARG, "loff must be >= 0");
-    hipLaunchKernelGGL(rope_kernel, dim3(num_heads), dim3(head_size / 2), 0, ctx->stream, q, k, num_kv_heads, head_size, pos,
+    awq_launch(ctx, rope_kernel, dim3(num_heads), dim3(head_size / 2), 0, q, k, num_kv_heads, head_size, pos,
                        loff, rope_theta);
     return awq_check_launch("rope");
 }

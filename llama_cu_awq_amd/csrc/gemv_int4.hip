@@ -327,9 +327,9 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     const dim3 grid(gx, grid_y);
     const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
     if (p.norm_w)
-        hipLaunchKernelGGL((gemv_int4_kernel<W, R, D, KIND, true, ROPE>), grid, dim3(W * 64), lds, ctx->stream, p);
+        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, true, ROPE>, grid, dim3(W * 64), lds, p);
     else
-        hipLaunchKernelGGL((gemv_int4_kernel<W, R, D, KIND, false, ROPE>), grid, dim3(W * 64), lds, ctx->stream, p);
+        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, ROPE>, grid, dim3(W * 64), lds, p);
     return awq_check_launch(what);
 }
 

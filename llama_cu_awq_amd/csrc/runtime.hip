@@ -65,6 +65,7 @@ static int ctx_init(int device, hipStream_t stream, bool owns, awq_ctx** out) {
     c->device = device;
     c->stream = stream;
     c->owns_stream = owns;
+    c->probe = nullptr;
     c->gemm_part = nullptr;
     c->gemm_part_bytes = 0;
     c->gemm_counter = nullptr;

@@ -469,6 +469,16 @@ int network_reference(awq_transformer* t, int seq_len_bin) {
     return awq_matvec_f16(ctx, s.logits, s.x, t->wcls, dim, p.vocab_size);
 }
 
+// Launch kinds of the fused schedule, as awq_transformer_time_launches reports them.
+enum { LK_EMBED = 0, LK_QKV = 1, LK_ATTENTION = 2, LK_OPROJ = 3, LK_GATE_UP = 4, LK_DOWN = 5, LK_CLASSIFIER = 6, LK_COUNT = 7 };
+
+// Names the schedule step whose launches follow, for a timing run (see awq_launch in common.hpp); otherwise free.
+struct LaunchProbe {
+    LaunchProbe(awq_transformer* t, int kind) {
+        if (t->ctx->probe) t->ctx->probe->kind = kind;
+    }
+};
+
 // Same arithmetic with RMSNorm folded into the staging of the consuming
 // matrix-vector kernels (the normalised vector never travels through memory).
 int network_fused(awq_transformer* t, int seq_len_bin) {
@@ -482,33 +492,52 @@ int network_fused(awq_transformer* t, int seq_len_bin) {
     int* pPos = s.pos;
     int r;
     // the token list's device mirror (kept by reset / set_pos / accept / the sampler) saves a read over PCIe
-    if ((r = awq_embed(ctx, s.x, t->embed, dim, t->tokens_dev, pPos))) return r;
+    {
+        LaunchProbe probe(t, LK_EMBED);
+        if ((r = awq_embed(ctx, s.x, t->embed, dim, t->tokens_dev, pPos))) return r;
+    }
     for (int l = 0; l < p.n_layers; l++) {
         const awq_layer_weights& L = t->layers[l];
         const int loff = l * p.seq_len * kv_dim;
-        if (dim == kv_dim) {
-            if ((r = awq_launch_qkv(ctx, s.q, s.key_cache, s.value_cache, s.x, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, loff, pPos,
-                                    L.rms_att_weight, nullptr, t->rope_table, head_size)))
-                return r;
-        } else {
-            if ((r = awq_launch_matvec_int4(ctx, s.q, s.x, &L.wq_q, dim, dim, 0, 1, -1, nullptr, L.rms_att_weight, nullptr)))
-                return r;
-            if ((r = awq_launch_matvec_int4(ctx, s.key_cache, s.x, &L.wq_k, dim, kv_dim, 0, 1, loff, pPos, L.rms_att_weight,
-                                            nullptr)))
-                return r;
-            if ((r = awq_launch_matvec_int4(ctx, s.value_cache, s.x, &L.wq_v, dim, kv_dim, 0, 1, loff, pPos, L.rms_att_weight,
-                                            nullptr)))
-                return r;
-            if ((r = awq_rope(ctx, s.q, s.key_cache, p.n_heads, p.n_kv_heads, head_size, pPos, loff, p.rope_theta))) return r;
+        {
+            LaunchProbe probe(t, LK_QKV);
+            if (dim == kv_dim) {
+                if ((r = awq_launch_qkv(ctx, s.q, s.key_cache, s.value_cache, s.x, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, loff, pPos,
+                                        L.rms_att_weight, nullptr, t->rope_table, head_size)))
+                    return r;
+            } else {
+                if ((r = awq_launch_matvec_int4(ctx, s.q, s.x, &L.wq_q, dim, dim, 0, 1, -1, nullptr, L.rms_att_weight, nullptr)))
+                    return r;
+                if ((r = awq_launch_matvec_int4(ctx, s.key_cache, s.x, &L.wq_k, dim, kv_dim, 0, 1, loff, pPos, L.rms_att_weight,
+                                                nullptr)))
+                    return r;
+                if ((r = awq_launch_matvec_int4(ctx, s.value_cache, s.x, &L.wq_v, dim, kv_dim, 0, 1, loff, pPos, L.rms_att_weight,
+                                                nullptr)))
+                    return r;
+                if ((r = awq_rope(ctx, s.q, s.key_cache, p.n_heads, p.n_kv_heads, head_size, pPos, loff, p.rope_theta))) return r;
+            }
         }
-        if ((r = awq_attention(ctx, s.xb, s.q, s.key_cache + loff, s.value_cache + loff, s.att, p.n_heads, head_size, kv_mul,
-                               seq_len_bin, pPos)))
-            return r;
-        if ((r = awq_launch_matvec_int4(ctx, s.x, s.xb, &L.wq_o, dim, dim, 1, 1, -1, nullptr, nullptr, nullptr))) return r;
-        if ((r = awq_launch_ffn(ctx, s.hb, s.x, &L.wq_gate, &L.wq_up, dim, hidden_dim, L.rms_ffn_weight, nullptr))) return r;
-        if ((r = awq_launch_matvec_int4(ctx, s.x, s.hb, &L.wq_down, hidden_dim, dim, 1, 1, -1, nullptr, nullptr, nullptr)))
-            return r;
+        {
+            LaunchProbe probe(t, LK_ATTENTION);
+            if ((r = awq_attention(ctx, s.xb, s.q, s.key_cache + loff, s.value_cache + loff, s.att, p.n_heads, head_size, kv_mul,
+                                   seq_len_bin, pPos)))
+                return r;
+        }
+        {
+            LaunchProbe probe(t, LK_OPROJ);
+            if ((r = awq_launch_matvec_int4(ctx, s.x, s.xb, &L.wq_o, dim, dim, 1, 1, -1, nullptr, nullptr, nullptr))) return r;
+        }
+        {
+            LaunchProbe probe(t, LK_GATE_UP);
+            if ((r = awq_launch_ffn(ctx, s.hb, s.x, &L.wq_gate, &L.wq_up, dim, hidden_dim, L.rms_ffn_weight, nullptr))) return r;
+        }
+        {
+            LaunchProbe probe(t, LK_DOWN);
+            if ((r = awq_launch_matvec_int4(ctx, s.x, s.hb, &L.wq_down, hidden_dim, dim, 1, 1, -1, nullptr, nullptr, nullptr)))
+                return r;
+        }
     }
+    LaunchProbe probe(t, LK_CLASSIFIER);
     return awq_launch_matvec_f16(ctx, s.logits, s.x, t->wcls, dim, p.vocab_size, t->rms_final, nullptr);
 }
 
@@ -898,6 +927,43 @@ int awq_transformer_sample(awq_transformer* t, awq_sampler* sampler, int gen_tok
     AWQ_REQUIRE(t->issued_pos + 1 <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
     if (int r = awq_sampler_run(sampler, t->s.logits, t->s.shared_tokens, t->s.shared_pos, t->s.pos, gen_token, t->tokens_dev)) return r;
     t->issued_pos++;
+    return AWQ_OK;
+}
+
+int awq_transformer_time_launches(awq_transformer* t, int passes, float* us_by_kind, int* launches_by_kind) {
+    AWQ_REQUIRE(t && us_by_kind && launches_by_kind, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(passes >= 1 && passes <= 64, AWQ_ERR_ARG, "passes must be 1 .. 64");
+    awq_ctx* ctx = t->ctx;
+    if (int r = awq_bind(ctx)) return r;
+    const int seq_len = t->issued_pos + 1;
+    AWQ_REQUIRE(seq_len <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+    awq_launch_probe probe;
+    int r = network_fused(t, seq_len);  // untimed: code objects loaded, caches in their steady state
+    ctx->probe = &probe;
+    for (int i = 0; i < passes && r == AWQ_OK; i++) r = network_fused(t, seq_len);
+    ctx->probe = nullptr;
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    double sum[LK_COUNT] = {0};
+    int count[LK_COUNT] = {0};
+    if (r == AWQ_OK && e == hipSuccess) {
+        for (size_t i = 0; i < probe.kinds.size(); i++) {
+            float ms = 0.0f;
+            if (hipEventElapsedTime(&ms, probe.events[2 * i], probe.events[2 * i + 1]) == hipSuccess) {
+                sum[probe.kinds[i]] += ms * 1e3;
+                count[probe.kinds[i]]++;
+            }
+        }
+    }
+    for (hipEvent_t ev : probe.events) (void)hipEventDestroy(ev);
+    if (r) return r;
+    if (e != hipSuccess) {
+        awq_set_error("timing run failed: %s", hipGetErrorString(e));
+        return AWQ_ERR_HIP;
+    }
+    for (int k = 0; k < LK_COUNT; k++) {
+        us_by_kind[k] = count[k] ? (float)(sum[k] / count[k]) : 0.0f;
+        launches_by_kind[k] = count[k];
+    }
     return AWQ_OK;
 }
 

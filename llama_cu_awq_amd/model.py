@@ -74,6 +74,15 @@ class Transformer:
         """Record the launch sequences of every sequence-length bin below max_positions ahead of time."""
         check(lib.awq_transformer_capture(self.h, mode, max_positions))
 
+    LAUNCH_KINDS = ("embed", "qkv", "attention", "oproj", "gate_up", "down", "classifier")
+
+    def time_launches(self, passes=4):
+        """Mean GPU microseconds per launch of the fused schedule at the current position, by launch kind."""
+        us = (C.c_float * len(self.LAUNCH_KINDS))()
+        n = (C.c_int * len(self.LAUNCH_KINDS))()
+        check(lib.awq_transformer_time_launches(self.h, passes, us, n))
+        return {k: {"us": round(us[i], 3), "launches": n[i]} for i, k in enumerate(self.LAUNCH_KINDS)}
+
     def forward_logits(self, use_graph=False, mode=SCHEDULE_FUSED):
         """run_llama_network() alone: this position's logits, no sampler."""
         check(lib.awq_transformer_forward_logits(self.h, int(use_graph), mode))
