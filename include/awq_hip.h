@@ -133,6 +133,20 @@ int awq_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const uint1
                   const uint16_t* value_cache, uint16_t* att, int num_heads, int head_size, int kv_mul,
                   int max_seq_len, const int* pos);
 
+/* The two halves of MultiHeadAttention + the O projection (llama2_q4.cu:410-427, 487) as the fused schedule runs them
+ * at long contexts.  awq_attention_partial: scores as awq_attention, then the probability-weighted sum of the value
+ * rows split over `*chunks` contiguous ranges of positions (chosen by the library, at most AWQ_ATTENTION_MAX_CHUNKS),
+ * written as fp32 partial sums part[chunk][num_heads * head_size]; the probabilities are the reference's (softmax over
+ * all positions, rounded to fp16).  awq_matvec_int4_parts: out = half(W x [+ out]) where x = half(part[0] + part[1] +
+ * ... ) is formed while the input vector is staged (the reference's fp16 rounding of the attention output).
+ * part: AWQ_ATTENTION_MAX_CHUNKS * num_heads * head_size floats.  K <= 8192. */
+#define AWQ_ATTENTION_MAX_CHUNKS 4
+int awq_attention_partial(awq_ctx* ctx, float* part, int* chunks, const uint16_t* q, const uint16_t* key_cache,
+                          const uint16_t* value_cache, uint16_t* att, int num_heads, int head_size, int kv_mul, int max_seq_len,
+                          const int* pos);
+int awq_matvec_int4_parts(awq_ctx* ctx, uint16_t* out, const float* part, int parts, const awq_qweight* w, int K, int N,
+                          int accum);
+
 /* matmul(half), llama2_q4.cu:357-365 as used for the classifier (:530): out[r] = half(sum_j w[r*n+j] x[j]),
  * w row-major (d, n).  The batch/stride/alpha generality of the reference launcher is unused on its live path. */
 int awq_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d);

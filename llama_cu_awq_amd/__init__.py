@@ -6,6 +6,7 @@ from .ops import (  # noqa: F401
     QWeight,
     Sampler,
     MultiHeadAttention,
+    MultiHeadAttention_partial,
     RoPERotation,
     argmax_advance,
     copy_embedding,
@@ -15,6 +16,7 @@ from .ops import (  # noqa: F401
     gemm_q_static,
     matmul,
     matmul_q,
+    matmul_q_parts,
     qkv_matvec,
     rmsnorm,
     rmsnorm_ffn_matvec_silu,

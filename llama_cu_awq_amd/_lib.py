@@ -67,6 +67,8 @@ PROTOTYPES = {
     "awq_rmsnorm_ffn_matvec_silu": [_vp, _vp, _vp, _vp, _pq, _pq, _i, _i],
     "awq_rope": [_vp, _vp, _vp, _i, _i, _i, _vp, _i, _f],
     "awq_attention": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "awq_attention_partial": [_vp, _vp, C.POINTER(C.c_int), _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "awq_matvec_int4_parts": [_vp, _vp, _vp, _i, _pq, _i, _i, _i],
     "awq_matvec_f16": [_vp, _vp, _vp, _vp, _i, _i],
     "awq_argmax_advance": [_vp, _vp, _i, _vp, _vp, _vp, _i],
     "awq_dequant": [_vp, _vp, _pq, _i, _i],

@@ -233,6 +233,126 @@ __global__ __launch_bounds__(1024) void attn_pv_sliced_kernel(uint16_t* output, 
     }
 }
 
+// Long contexts in the fused schedule: P.V split over positions as well, so that every compute unit pulls whole
+// cache lines.  A workgroup of 16 waves owns one head, one of `chunks` contiguous ranges of positions and one slice of
+// 64 value dimensions (128 bytes of every row: 8 lanes x 16 bytes); it computes the softmax statistics over ALL
+// positions from the fp16 scores (as every workgroup of the head does, in the same order, so they agree bit for bit),
+// forms the fp16-rounded probabilities of its own positions exactly as the reference does (gpu_kernels.h:376-409) and
+// writes the fp32 sum of p * v over its range to part[chunk][head * head_size + dim].  The chunks of a head are added
+// up, in chunk order, by the consumer (the O projection's staging), where the sum is rounded to fp16: the rounding
+// point of the reference's attention output.  No exchange between workgroups, no atomics, one launch.
+constexpr int kPvPartialRows = 8;  // value rows in flight per thread
+
+__global__ __launch_bounds__(1024) void attn_pv_partial_kernel(float* part, const uint16_t* att, const uint16_t* value_cache,
+                                                              int head_size, int kv_mul, int row_stride, int chunks, int out_dim,
+                                                              const int* pPos) {
+    constexpr int R = kPvPartialRows;
+    __shared__ float red[16];
+    __shared__ float acc_lds[16][64];
+    const int size = *pPos + 1;
+    const int h = blockIdx.x, chunk = blockIdx.y, slice = blockIdx.z;
+    const int per = (size + chunks - 1) / chunks;
+    const int t_begin = chunk * per, t_end = min(size, t_begin + per);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rg = tid >> 3, ql = tid & 7;  // row group (128 rows per pass), 16-byte piece of the slice
+    const uint16_t* a = att + (size_t)h * size;
+    const uint16_t* vh = value_cache + (size_t)(h / kv_mul) * head_size + slice * 64 + ql * 8;
+    u32x4 vv[R];
+    uint16_t sv[R];
+    // Loads return in order: the scores that the statistics need (two per thread cover 2048 positions) are requested
+    // ahead of the value rows, so that the statistics are computed while the rows are still on their way.
+    uint16_t stat[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+        if (tid + 1024 * j < size) stat[j] = a[tid + 1024 * j];
+    auto request = [&](int t0) {
+#pragma unroll
+        for (int k = 0; k < R; k++) {
+            const int t = t0 + rg + 128 * k;
+            if (t < t_end) sv[k] = a[t];
+        }
+#pragma unroll
+        for (int k = 0; k < R; k++) {
+            const int t = t0 + rg + 128 * k;
+            if (t < t_end) vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+        }
+    };
+    request(t_begin);
+    // statistics over all positions (the max seed is the reference's idle-lane 0 when its 1024-thread block is not full)
+    float m = (size < 1024) ? 0.0f : -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+        if (tid + 1024 * j < size) m = fmaxf(m, half_bits_to_float(stat[j]));
+    for (int t = tid + 2048; t < size; t += 1024) m = fmaxf(m, half_bits_to_float(a[t]));
+    m = wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < 16; w++) m = fmaxf(m, red[w]);
+    __syncthreads();
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+        if (tid + 1024 * j < size) sum += expf(half_bits_to_float(stat[j]) - m);
+    for (int t = tid + 2048; t < size; t += 1024) sum += expf(half_bits_to_float(a[t]) - m);
+    sum = wave_sum(sum);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    {
+        float r[16];
+#pragma unroll
+        for (int w = 0; w < 16; w++) r[w] = red[w];
+#pragma unroll
+        for (int n = 16; n > 1; n >>= 1)
+#pragma unroll
+            for (int i = 0; i < n / 2; i++) r[i] = r[2 * i] + r[2 * i + 1];
+        sum = r[0];
+    }
+
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.0f;
+    for (int t0 = t_begin; t0 < t_end; t0 += 128 * R) {
+        if (t0 != t_begin) request(t0);
+#pragma unroll
+        for (int k = 0; k < R; k++) {
+            const int t = t0 + rg + 128 * k;
+            if (t < t_end) {
+                const float e = expf(half_bits_to_float(sv[k]) - m);
+                const float p = half_bits_to_float(float_to_half_bits(e / sum));  // probability rounded to fp16
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const h16x2 hv = as_h2(vv[k][i]);
+                    acc[2 * i] = fmaf((float)hv[0], p, acc[2 * i]);
+                    acc[2 * i + 1] = fmaf((float)hv[1], p, acc[2 * i + 1]);
+                }
+            }
+        }
+    }
+    // the 8 row groups of a wave (lanes with the same lane % 8), then the 16 waves
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        acc[i] = lane_xor_sum<8>(acc[i]);
+        acc[i] = lane_xor_sum<16>(acc[i]);
+        acc[i] = lane_xor_sum<32>(acc[i]);
+    }
+    if (lane < 8) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc_lds[wave][lane * 8 + i] = acc[i];
+    }
+    __syncthreads();
+    if (tid < 64) {
+        float r[16];
+#pragma unroll
+        for (int w = 0; w < 16; w++) r[w] = acc_lds[w][tid];
+#pragma unroll
+        for (int n = 16; n > 1; n >>= 1)
+#pragma unroll
+            for (int i = 0; i < n / 2; i++) r[i] = r[2 * i] + r[2 * i + 1];
+        part[(size_t)chunk * out_dim + (size_t)h * head_size + slice * 64 + tid] = r[0];
+    }
+}
+
 // Short contexts: a workgroup of 16 waves does scores, softmax and P.V of a head in a single launch (the work is a few
 // hundred KB per head, so the launch count matters more than the parallelism); NS workgroups per head each take a
 // slice of the value dimensions and compute the scores redundantly.  Same arithmetic and
@@ -465,6 +585,33 @@ int awq_launch_argmax(awq_ctx* ctx, const uint16_t* logits, int size, int* token
     return awq_check_launch("argmax");
 }
 
+// Internal (fused schedule, launch sizes above kAttnFusedMaxSeq): scores, then P.V as fp32 partial sums over
+// `*chunks_out` ranges of positions, part[chunk][num_heads * head_size]; the consumer adds the chunks up in order and
+// rounds to fp16.  part must hold kAttnMaxChunks * num_heads * head_size floats.
+int awq_launch_attention_partial(awq_ctx* ctx, float* part, int* chunks_out, const uint16_t* q, const uint16_t* key_cache,
+                                 const uint16_t* value_cache, uint16_t* att, int num_heads, int head_size, int kv_mul,
+                                 int max_seq_len, const int* pos) {
+    const int row_stride = num_heads * head_size / kv_mul;
+    const float alpha = (float)(1.0 / sqrt((double)head_size));
+    const int slices = head_size / 64;
+    // about one workgroup per compute unit, each pulling whole cache lines
+    int chunks = 256 / (num_heads * slices);
+    if (chunks < 1) chunks = 1;
+    if (chunks > kAttnMaxChunks) chunks = kAttnMaxChunks;
+    const dim3 sgrid(div_up(max_seq_len, 64), num_heads);
+    switch (head_size) {
+        case 64: awq_launch(ctx, attn_scores_kernel<8>, sgrid, dim3(256), 0, att, q, key_cache, head_size, kv_mul, row_stride, alpha, pos); break;
+        case 128: awq_launch(ctx, attn_scores_kernel<16>, sgrid, dim3(256), 0, att, q, key_cache, head_size, kv_mul, row_stride, alpha, pos); break;
+        case 256: awq_launch(ctx, attn_scores_kernel<32>, sgrid, dim3(256), 0, att, q, key_cache, head_size, kv_mul, row_stride, alpha, pos); break;
+        default: awq_set_error("attention: head_size %d unsupported (64, 128 or 256)", head_size); return AWQ_ERR_SHAPE;
+    }
+    if (int r = awq_check_launch("attn_scores")) return r;
+    awq_launch(ctx, attn_pv_partial_kernel, dim3(num_heads, chunks, slices), dim3(1024), 0, part, att, value_cache, head_size, kv_mul,
+               row_stride, chunks, num_heads * head_size, pos);
+    *chunks_out = chunks;
+    return awq_check_launch("attn_pv_partial");
+}
+
 // Internal: fp16 matvec with optional fused RMSNorm of x (norm_out must not alias x).
 int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
                           const uint16_t* norm_w, uint16_t* norm_out) {
@@ -526,6 +673,19 @@ int awq_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const uint1
             awq_set_error("awq_attention: head_size %d unsupported (64, 128 or 256)", head_size);
             return AWQ_ERR_SHAPE;
     }
+}
+
+int awq_attention_partial(awq_ctx* ctx, float* part, int* chunks, const uint16_t* q, const uint16_t* key_cache,
+                          const uint16_t* value_cache, uint16_t* att, int num_heads, int head_size, int kv_mul, int max_seq_len,
+                          const int* pos) {
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(part && chunks && q && key_cache && value_cache && att && pos, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(num_heads > 0 && num_heads <= kAttnMaxHeads, AWQ_ERR_SHAPE, "num_heads out of range");
+    AWQ_REQUIRE(kv_mul > 0 && num_heads % kv_mul == 0, AWQ_ERR_SHAPE, "kv_mul must divide num_heads");
+    AWQ_REQUIRE(max_seq_len > 0, AWQ_ERR_SHAPE, "max_seq_len must be positive");
+    static_assert(kAttnMaxChunks == AWQ_ATTENTION_MAX_CHUNKS, "header and library disagree");
+    return awq_launch_attention_partial(ctx, part, chunks, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len,
+                                        pos);
 }
 
 int awq_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d) {

@@ -13,7 +13,10 @@ struct XArgs {
     uint16_t* norm_out;      // optional: workgroup (0, 0) also stores the normalised vector here
     int K;
     int C;                   // 32-element chunks = ceil(K / 32)
+    const float* part;       // PARTS form: x = half(part[0][k] + part[1][k] + ...), rows K floats apart
+    int parts;               // 1 .. kMaxParts
 };
+constexpr int kMaxParts = 4;
 
 // 2^-24 * sum over the 32 consecutive K elements of one chunk of (q - z) * x.
 //
@@ -78,6 +81,65 @@ __device__ __forceinline__ void load_x(XPieces<NORM>& xr, const XArgs& p) {
         const int e = min(i * T + (int)threadIdx.x, n8 - 1);  // clamped, masked in stage_x
         xr.v[i] = xg[e];
         if (NORM) xr.w[i] = wg[e];
+    }
+}
+
+// The PARTS form of load_x: the activation vector arrives as up to kMaxParts fp32 partial sums per element (the
+// chunks of the position-split attention); their sum, added in part order and rounded to fp16 once, is x.  The loads
+// are requested here, ahead of the packed weights; combine_x turns them into the pieces stage_x takes.
+struct PartPieces {
+    u32x4 f[XP][kMaxParts][2];  // 8 floats per piece and part
+};
+
+template <int W>
+__device__ __forceinline__ void load_parts(PartPieces& pr, const XArgs& p) {
+    constexpr int T = W * 64;
+    const int n8 = p.K >> 3;
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        if (i > 0 && i * T >= n8) break;
+        const int e = min(i * T + (int)threadIdx.x, n8 - 1);
+#pragma unroll
+        for (int s = 0; s < kMaxParts; s++) {
+            if (s >= p.parts) break;  // uniform
+            const u32x4* src = reinterpret_cast<const u32x4*>(p.part + (size_t)s * p.K) + 2 * e;
+            pr.f[i][s][0] = src[0];
+            pr.f[i][s][1] = src[1];
+        }
+    }
+}
+
+template <int W>
+__device__ __forceinline__ void combine_x(XPieces<false>& xr, const PartPieces& pr, const XArgs& p) {
+    constexpr int T = W * 64;
+    const int n8 = p.K >> 3;
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        if (i > 0 && i * T >= n8) break;
+        // (a vector element goes through a scalar before the bit cast: cast directly, the element reference is
+        // taken as the vector's storage and every lane of it reads element 0)
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t u = pr.f[i][0][j >> 2][j & 3];
+            v[j] = __builtin_bit_cast(float, u);
+        }
+#pragma unroll
+        for (int s = 1; s < kMaxParts; s++) {
+            if (s >= p.parts) break;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t u = pr.f[i][s][j >> 2][j & 3];
+                v[j] += __builtin_bit_cast(float, u);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            h16x2 o;
+            o[0] = (h16_t)v[2 * j];
+            o[1] = (h16_t)v[2 * j + 1];
+            xr.v[i][j] = as_u32(o);
+        }
     }
 }
 

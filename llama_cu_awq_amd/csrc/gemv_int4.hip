@@ -46,6 +46,8 @@ struct GemvParams {
     const int* pos;
     const float2* rope;      // fused RoPE: (cos, sin) table [position][head_size/2], or null
     int head_size;           // for the fused RoPE row pairing
+    const float* xpart;      // PARTS form: x is the sum of `xparts` fp32 vectors K floats apart, rounded to fp16
+    int xparts;
 };
 
 enum { KIND_SINGLE = 0, KIND_QKV = 1, KIND_FFN = 2 };
@@ -60,8 +62,9 @@ __device__ __forceinline__ int map_row(int li, int head_size) {
     return (pi / half) * head_size + (pi % half) + (li & 1) * half;
 }
 
-template <int W, int R, int D, int KIND, bool NORM, bool ROPE>
+template <int W, int R, int D, int KIND, bool NORM, bool ROPE, bool PARTS = false>
 __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
+    static_assert(!PARTS || (!NORM && KIND == KIND_SINGLE), "partial-sum input only for the plain single-matrix form");
     extern __shared__ u32x4 xs[];
     __shared__ float red[W + 1];
     const int lane = threadIdx.x & 63;
@@ -222,13 +225,18 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
 
     // The first D stages of packed weights are requested before x is staged, so that their HBM latency overlaps the
     // staging (and the RMSNorm reduction).
-    const XArgs xa{p.x, p.norm_w, p.norm_out, p.K, p.C};
+    const XArgs xa{p.x, p.norm_w, p.norm_out, p.K, p.C, p.xpart, p.xparts};
     XPieces<NORM> xr;
-    load_x<W, NORM>(xr, xa);
+    PartPieces pr;
+    if constexpr (PARTS)
+        load_parts<W>(pr, xa);
+    else
+        load_x<W, NORM>(xr, xa);
     Stage<NS> st[D];
     set_rows(lg);
 #pragma unroll
     for (int d = 0; d < D; d++) issue(st[d]);
+    if constexpr (PARTS) combine_x<W>(xr, pr, xa);
     stage_x<W, NORM>(xs, ca, xa, red, xr);
     const int rounds = (total + D - 1) / D;
     for (int r = 1; r < rounds; r++) {
@@ -293,6 +301,8 @@ void fill_common(GemvParams& p, const uint16_t* x, int K, int N) {
     p.pos = nullptr;
     p.rope = nullptr;
     p.head_size = 0;
+    p.xpart = nullptr;
+    p.xparts = 0;
 }
 
 Int4Mat to_mat(const awq_qweight* w) { return Int4Mat{w->weight, w->zeros, w->scales}; }
@@ -326,6 +336,16 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     }
     const dim3 grid(gx, grid_y);
     const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
+    if constexpr (KIND == KIND_SINGLE && !ROPE && R == 1 && (W == 8 || W == 16)) {
+        if (p.xpart) {
+            awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, false, true>, grid, dim3(W * 64), lds, p);
+            return awq_check_launch(what);
+        }
+    }
+    if (p.xpart) {
+        awq_set_error("%s: no kernel takes partial-sum input in this geometry", what);
+        return AWQ_ERR_ARG;
+    }
     if (p.norm_w)
         awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, true, ROPE>, grid, dim3(W * 64), lds, p);
     else
@@ -392,6 +412,23 @@ int awq_launch_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const
     return dispatch<KIND_SINGLE, false>(ctx, p, 1, "gemv_int4", plan_for(K, 1));
 }
 
+// out = half(W x [+ out]) with x = half(part[0] + part[1] + ...): the O projection behind the position-split attention.
+int awq_launch_matvec_int4_parts(awq_ctx* ctx, uint16_t* out, const float* part, int parts, const awq_qweight* w, int K, int N,
+                                 int accum) {
+    if (parts < 1 || parts > kMaxParts || K > XP * 8 * 64 * 8) {  // every piece of x travels in registers (8-wave workgroups)
+        awq_set_error("matvec with partial-sum input: %d parts, K = %d not supported", parts, K);
+        return AWQ_ERR_SHAPE;
+    }
+    GemvParams p;
+    fill_common(p, nullptr, K, N);
+    p.m[0] = to_mat(w);
+    p.out[0] = out;
+    p.accum = accum;
+    p.xpart = part;
+    p.xparts = parts;
+    return dispatch<KIND_SINGLE, false>(ctx, p, 1, "gemv_int4_parts", plan_for(K, 1));
+}
+
 int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
                    const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw, int K, int N, int loff,
                    const int* pos, const uint16_t* norm_w, uint16_t* norm_out, const float2* rope, int head_size) {
@@ -454,6 +491,14 @@ int awq_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const aw
     if (int r = check_shape(K, N)) return r;
     AWQ_REQUIRE(out && x && qw_ok(gate_w) && qw_ok(up_w), AWQ_ERR_ARG, "null pointer");
     return awq_launch_ffn(ctx, out, x, gate_w, up_w, K, N, nullptr, nullptr);
+}
+
+int awq_matvec_int4_parts(awq_ctx* ctx, uint16_t* out, const float* part, int parts, const awq_qweight* w, int K, int N,
+                          int accum) {
+    if (int r = awq_bind(ctx)) return r;
+    if (int r = check_shape(K, N)) return r;
+    AWQ_REQUIRE(out && part && qw_ok(w), AWQ_ERR_ARG, "null pointer");
+    return awq_launch_matvec_int4_parts(ctx, out, part, parts, w, K, N, accum);
 }
 
 int awq_rmsnorm_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* norm_weight,

@@ -23,6 +23,11 @@ int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qwe
                    int N, const uint16_t* norm_w, uint16_t* norm_out);
 int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
                           const uint16_t* norm_w, uint16_t* norm_out);
+int awq_launch_attention_partial(awq_ctx* ctx, float* part, int* chunks_out, const uint16_t* q, const uint16_t* key_cache,
+                                 const uint16_t* value_cache, uint16_t* att, int num_heads, int head_size, int kv_mul,
+                                 int max_seq_len, const int* pos);
+int awq_launch_matvec_int4_parts(awq_ctx* ctx, uint16_t* out, const float* part, int parts, const awq_qweight* w, int K, int N,
+                                 int accum);
 int awq_launch_argmax(awq_ctx* ctx, const uint16_t* logits, int size, int* tokens, volatile int* pos_host, int* pos_dev,
                       int write_token, int* tokens_mirror);
 // sampler.hip
@@ -100,6 +105,7 @@ struct awq_transformer {
     bool captured[2][kMaxGraphs];
     int* tokens_dev;  // device mirror of SharedData.tokens (the persistent kernel reads its input token here)
     float2* rope_table;  // [seq_len][head_size/2] (cos, sin)
+    float* attn_part;    // [kAttnMaxChunks][dim] fp32 partial attention outputs of the position-split form
     // plan of the persistent per-token kernel
     bool tk_ok;
     char tk_why[160];  // why the persistent kernel cannot run this model, when !tk_ok
@@ -206,6 +212,7 @@ int alloc_state(awq_transformer* t) {
     AWQ_HIP_TRY(hipMemset(t->tokens_dev, 0, (size_t)(c.seq_len + 8) * sizeof(int)));
     const int head = c.dim / c.n_heads;
     AWQ_HIP_TRY(hipMalloc((void**)&t->rope_table, (size_t)c.seq_len * (head / 2) * sizeof(float2)));
+    AWQ_HIP_TRY(hipMalloc((void**)&t->attn_part, (size_t)kAttnMaxChunks * c.dim * sizeof(float)));
     hipLaunchKernelGGL(rope_table_kernel, dim3(c.seq_len), dim3(head / 2), 0, t->ctx->stream, t->rope_table, head / 2, head, c.rope_theta);
     if (int r = awq_check_launch("rope_table")) return r;
     s.shared_pos = &t->shared->pos;
@@ -231,6 +238,7 @@ void release(awq_transformer* t) {
     if (t->shared) (void)hipHostFree(t->shared);
     (void)hipFree(t->tokens_dev);
     (void)hipFree(t->rope_table);
+    (void)hipFree(t->attn_part);
     (void)hipFree(t->tk_phases);
     (void)hipFree(t->tk_sync);
     (void)hipFree(t->tk_trace);
@@ -251,6 +259,7 @@ awq_transformer* new_transformer(awq_ctx* ctx) {
     t->shared = nullptr;
     t->tokens_dev = nullptr;
     t->rope_table = nullptr;
+    t->attn_part = nullptr;
     t->tk_ok = false;
     t->tk_why[0] = 0;
     t->tk_phases = nullptr;
@@ -517,15 +526,27 @@ int network_fused(awq_transformer* t, int seq_len_bin) {
                 if ((r = awq_rope(ctx, s.q, s.key_cache, p.n_heads, p.n_kv_heads, head_size, pPos, loff, p.rope_theta))) return r;
             }
         }
+        // Long launch sizes: P.V split over positions too, its fp32 partial sums added up (and rounded to fp16, the
+        // reference's rounding point) while the O projection stages its input; xb is not written on this path.
+        const bool split = seq_len_bin > kAttnFusedMaxSeq && dim <= 8192;
+        int parts = 0;
         {
             LaunchProbe probe(t, LK_ATTENTION);
-            if ((r = awq_attention(ctx, s.xb, s.q, s.key_cache + loff, s.value_cache + loff, s.att, p.n_heads, head_size, kv_mul,
-                                   seq_len_bin, pPos)))
-                return r;
+            if (split)
+                r = awq_launch_attention_partial(ctx, t->attn_part, &parts, s.q, s.key_cache + loff, s.value_cache + loff, s.att,
+                                                 p.n_heads, head_size, kv_mul, seq_len_bin, pPos);
+            else
+                r = awq_attention(ctx, s.xb, s.q, s.key_cache + loff, s.value_cache + loff, s.att, p.n_heads, head_size, kv_mul,
+                                  seq_len_bin, pPos);
+            if (r) return r;
         }
         {
             LaunchProbe probe(t, LK_OPROJ);
-            if ((r = awq_launch_matvec_int4(ctx, s.x, s.xb, &L.wq_o, dim, dim, 1, 1, -1, nullptr, nullptr, nullptr))) return r;
+            if (split)
+                r = awq_launch_matvec_int4_parts(ctx, s.x, t->attn_part, parts, &L.wq_o, dim, dim, 1);
+            else
+                r = awq_launch_matvec_int4(ctx, s.x, s.xb, &L.wq_o, dim, dim, 1, 1, -1, nullptr, nullptr, nullptr);
+            if (r) return r;
         }
         {
             LaunchProbe probe(t, LK_GATE_UP);

@@ -181,6 +181,23 @@ def MultiHeadAttention(ctx, output, q, key_cache, value_cache, att, num_heads, h
     )
 
 
+def MultiHeadAttention_partial(ctx, part, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pPos):
+    """Scores + position-split P.V (fp32 partial sums per range of positions); returns the number of ranges."""
+    n = C.c_int()
+    check(
+        lib.awq_attention_partial(
+            ctx.h, _addr(part), C.byref(n), _addr(q), _addr(key_cache), _addr(value_cache), _addr(att), num_heads, head_size,
+            kv_mul, max_seq_len, _addr(pPos),
+        )
+    )
+    return n.value
+
+
+def matmul_q_parts(ctx, xout, part, parts, w, inpSize, opSize, accum=False):
+    """matmul(QWeight) whose input vector is half(sum of `parts` fp32 vectors) (the O projection behind the split attention)."""
+    check(lib.awq_matvec_int4_parts(ctx.h, _addr(xout), _addr(part), parts, C.byref(w.c), inpSize, opSize, int(accum)))
+
+
 def argmax_advance(ctx, logits, size, tokens, pos_host, pos_dev, write_token):
     """sample() greedy branch, sampler.h:77-84."""
     check(lib.awq_argmax_advance(ctx.h, _addr(logits), size, _addr(tokens), _addr(pos_host), _addr(pos_dev), int(write_token)))

@@ -286,6 +286,49 @@ def test_attention(ctx, heads, head, kv_mul, pos, max_seq):
     assert np.array_equal(dout.download(np.uint16), got.view(np.uint16))
 
 
+@pytest.mark.parametrize(
+    "heads,head,kv_mul,pos,max_seq",
+    [(32, 128, 1, 256, 257), (32, 128, 1, 271, 512), (40, 128, 1, 1791, 2048), (52, 128, 1, 2047, 2048), (8, 64, 4, 300, 512), (4, 256, 2, 1023, 1024), (32, 128, 1, 2, 512)],
+)
+def test_attention_split_over_positions_then_o_projection(ctx, heads, head, kv_mul, pos, max_seq):
+    """The long-context form of the fused schedule: P.V as fp32 partial sums per range of positions, added up and
+    rounded to fp16 inside the O projection's staging.  The rounded sum of the partials must be the attention output
+    (same probabilities, only the fp32 order of the sum over positions differs), and the product taken from the
+    partials must be the product of that vector."""
+    kv_dim, dim = heads * head // kv_mul, heads * head
+    seq = pos + 1
+    key = synth.stream_key(55, heads, head, kv_mul, pos)
+    q = synth.normal_f16(synth.stream_key(key, "q"), dim)
+    kc = synth.normal_f16(synth.stream_key(key, "k"), seq * kv_dim)
+    vc = synth.normal_f16(synth.stream_key(key, "v"), seq * kv_dim)
+    dq, dk, dv = ctx.upload(q), ctx.upload(kc), ctx.upload(vc)
+    datt = ctx.zeros(heads * max(max_seq, seq) * 2)
+    dpos = ctx.upload(np.array([pos], dtype=np.int32))
+    dpart = ctx.upload(np.full(4 * dim, np.nan, dtype=np.float32))  # whatever the chunks do not write would poison the sum
+    chunks = A.MultiHeadAttention_partial(ctx, dpart, dq, dk, dv, datt, heads, head, kv_mul, max_seq, dpos)
+    assert 1 <= chunks <= 4
+    part = dpart.download(np.float32).reshape(4, dim)[:chunks]
+    acc = part[0].copy()
+    for c in range(1, chunks):
+        acc = acc + part[c]  # fp32, chunk order: what the consumer does
+    got = acc.astype(np.float16)
+    want, want_att = oracle.attention(q, kc.view(np.uint16), vc.view(np.uint16), heads, head, kv_mul, pos)
+    assert rel_l2(got, want) <= 1.5e-3
+    dout = ctx.zeros(dim * 2)
+    A.MultiHeadAttention(ctx, dout, dq, dk, dv, datt, heads, head, kv_mul, max_seq, dpos)
+    assert_close_f16(got, f16(dout.download(np.uint16)), ulps=2)
+    # the O projection fed with the partials == the O projection fed with their rounded sum
+    if dim <= 8192:
+        N = 256
+        w, z, sc, _ = _case(dim, N, 56)
+        qw = A.QWeight.upload(ctx, w, z, sc)
+        resid = synth.normal_f16(synth.stream_key(key, "r"), N)
+        d1, d2 = ctx.upload(resid), ctx.upload(resid)
+        A.matmul_q_parts(ctx, d1, dpart, chunks, qw, dim, N, accum=True)
+        A.matmul_q(ctx, d2, ctx.upload(got), qw, dim, N, accum=True)
+        assert np.array_equal(d1.download(np.uint16), d2.download(np.uint16))
+
+
 def test_attention_pos0_returns_v0(ctx):
     heads, head = 32, 128
     q = synth.normal_f16(synth.stream_key(6, "q"), heads * head)
