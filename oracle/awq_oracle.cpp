@@ -547,6 +547,90 @@ int orc_sample_top_p(const uint16_t* probs, int size, float threshold, int sorte
     return token;
 }
 
+// The same selection with the prefix sum ADDED IN fp16, the arithmetic cub::DeviceScan::InclusiveSum performs on half
+// data (sampler.h:107-111): every partial sum is rounded to fp16, so the result depends on the order of the additions,
+// which CUB chooses and the reference does not fix.  Two orders a CUB scan can take are written out, to measure how
+// far the choice matters (neither is claimed to be the reference's):
+//   mode 0  strictly sequential: prefix[t] = half(prefix[t-1] + p[t]);
+//   mode 1  tiled, `threads` x `items` elements per tile: every thread adds up its `items` consecutive elements, the
+//           thread totals are scanned across each 32-lane group in log steps (lane i takes lane i - off, off = 1, 2,
+//           4, 8, 16), the group totals and the tile totals are carried forward sequentially, and each thread then
+//           scans its elements again starting from the sum of everything before them.
+// Returns the picked token; no position is advanced.
+static inline uint16_t hadd(uint16_t a, uint16_t b) { return f2h(h2f(a) + h2f(b)); }  // fp32 holds the exact sum's rounding: innocuous
+int orc_top_p_pick_fp16_scan(const uint16_t* probs, int size, float threshold, int sorted, int mode, int threads, int items) {
+    int* idx = (int*)malloc(sizeof(int) * (size_t)size);
+    for (int i = 0; i < size; i++) idx[i] = i;
+    if (sorted) {
+        int* count = (int*)calloc(65537, sizeof(int));
+        for (int i = 0; i < size; i++) count[65535 - probs[i]]++;
+        int run = 0;
+        for (int k = 0; k < 65536; k++) { int c = count[k]; count[k] = run; run += c; }
+        for (int i = 0; i < size; i++) idx[count[65535 - probs[i]]++] = i;
+        free(count);
+    }
+    uint16_t* prefix = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)size);
+    if (mode == 0) {
+        uint16_t run = 0;
+        for (int t = 0; t < size; t++) { run = t ? hadd(run, probs[idx[t]]) : probs[idx[t]]; prefix[t] = run; }
+    } else {
+        const int tile = threads * items;
+        uint16_t* total = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)threads);
+        uint16_t* excl = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)threads);
+        char* has = (char*)malloc((size_t)threads);  // thread owns at least one element
+        uint16_t carry = 0;  // sum of all earlier tiles
+        bool have_carry = false;
+        for (int base = 0; base < size; base += tile) {
+            for (int th = 0; th < threads; th++) {
+                const int b = base + th * items, e = b + items < size ? b + items : size;
+                has[th] = b < size;
+                uint16_t r = 0;
+                for (int t = b; t < e; t++) r = t == b ? probs[idx[t]] : hadd(r, probs[idx[t]]);
+                total[th] = r;
+            }
+            // inclusive scan of the thread totals inside each group of 32, log steps
+            for (int g = 0; g < threads; g += 32) {
+                const int n = threads - g < 32 ? threads - g : 32;
+                for (int off = 1; off < 32; off <<= 1) {
+                    uint16_t prev[32];
+                    for (int l = 0; l < n; l++) prev[l] = total[g + l];
+                    for (int l = off; l < n; l++)
+                        if (has[g + l]) total[g + l] = hadd(prev[l - off], prev[l]);
+                }
+            }
+            // exclusive prefix of every thread: earlier tiles + earlier groups + earlier lanes of its group
+            uint16_t groups = carry;
+            bool have_groups = have_carry;
+            for (int g = 0; g < threads; g += 32) {
+                const int n = threads - g < 32 ? threads - g : 32;
+                for (int l = 0; l < n; l++) {
+                    if (l == 0) excl[g] = groups;
+                    else excl[g + l] = have_groups ? hadd(groups, total[g + l - 1]) : total[g + l - 1];
+                }
+                int last = -1;
+                for (int l = 0; l < n; l++) if (has[g + l]) last = l;
+                if (last >= 0) { groups = have_groups ? hadd(groups, total[g + last]) : total[g + last]; have_groups = true; }
+            }
+            for (int th = 0; th < threads; th++) {
+                const int b = base + th * items, e = b + items < size ? b + items : size;
+                const bool seeded = (th % 32 != 0) || (th >= 32) || have_carry;
+                uint16_t r = excl[th];
+                for (int t = b; t < e; t++) { r = (t == b && !seeded) ? probs[idx[t]] : hadd(r, probs[idx[t]]); prefix[t] = r; }
+            }
+            carry = groups;
+            have_carry = true;
+        }
+        free(total); free(excl); free(has);
+    }
+    int pick = size - 1;
+    for (int t = 0; t < size; t++)
+        if (h2f(prefix[t]) >= threshold) { pick = t; break; }
+    const int token = idx[pick];
+    free(prefix);
+    free(idx);
+    return token;
+}
+
 // ---------------------------------------------------------------- model image
 // Config = the 32-byte file header (common.h:15-24).
 typedef struct {

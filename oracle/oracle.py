@@ -41,6 +41,7 @@ def _load():
         "orc_random_f32": ([vp], f),
         "orc_softmax_logits": ([vp, i, f], None),
         "orc_sample_top_p": ([vp, i, f, i, vp, vp, vp], i),
+        "orc_top_p_pick_fp16_scan": ([vp, i, f, i, i, i, i], i),
         "orc_model_file_bytes": ([vp], C.c_size_t),
         "orc_model_open": ([vp, C.c_size_t], vp),
         "orc_model_close": ([vp], None),
@@ -164,6 +165,12 @@ def softmax_logits(logits, temperature):
 def sample_top_p(probs, threshold, sorted_, tokens, pos_host, pos_dev):
     pp = _c(probs.view(np.uint16), np.uint16)
     return lib.orc_sample_top_p(_p(pp), pp.size, float(threshold), int(sorted_), _p(tokens), _p(pos_host), _p(pos_dev))
+
+
+def top_p_pick_fp16_scan(probs, threshold, sorted_, mode, threads=128, items=16):
+    """The top-p pick when the prefix sum is added in fp16: mode 0 sequentially, mode 1 in tiles of threads x items."""
+    pp = _c(probs.view(np.uint16), np.uint16)
+    return lib.orc_top_p_pick_fp16_scan(_p(pp), pp.size, float(threshold), int(sorted_), int(mode), int(threads), int(items))
 
 
 class Model:
