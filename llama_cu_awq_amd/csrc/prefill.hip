@@ -44,6 +44,8 @@ struct GemmParams {
     // [position][pair]; row m of the GEMM is position rope_pos0 + m.  Null: no rotation.
     const float2* rope;
     int rope_pos0;
+    // FFN form: write the output with every 8 columns in the order (0,4,1,5,2,6,3,7), the order a permuted-A GEMM reads
+    int out_perm;
     uint16_t* out[3];
     long long ldo[3];       // output row stride in elements
     long long out_off[3];   // element offset of output row 0 (KV cache: loff + pos0 * kv_dim)
@@ -58,6 +60,9 @@ __device__ __forceinline__ u32x4 permute8(const u32x4 v) {
     o[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
     return o;
 }
+
+// Where element j of a group of 8 sits in that order: (0,4,1,5,2,6,3,7) holds j at ((j & 3) << 1) | (j >> 2).
+__device__ __forceinline__ int permuted_index(int c) { return (c & ~7) | ((c & 3) << 1) | ((c >> 2) & 1); }
 
 // 8 nibbles of one dword -> 8 dequantised fp16 weights in the order (w0,w4)(w1,w5)(w2,w6)(w3,w7).
 // magic = 0x64006400 held in a vector register: v_and_or_b32 takes no literal, and with the constant in a register
@@ -153,6 +158,12 @@ __device__ __forceinline__ u32x4 unpermute8(const u32x4 v) {
 //    ones with zero scales), so the number of loads between a request and its use is constant.
 // Workgroup ids are mapped so that the M tiles sharing a weight tile run on one XCD (ids go round-robin over the 8
 // XCDs), which reads the weights from HBM once.
+//
+// APERM: every 16-byte chunk of A holds its 8 activations in the order (0,4,1,5,2,6,3,7), the order in which a packed
+// dword dequantises.  Both MFMA operands contract over K, so any order they agree on gives the same products; with A
+// already in that order the weights go into the MFMA as they come out of the dequantisation.  The prefill path writes
+// its intermediate activations that way; the public entry points take A in natural order.
+template <bool APERM>
 __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];  // [A ring][W ring]; nothing else is in LDS
     constexpr uint32_t W_RING = A_STAGES * TILE_BYTES;
@@ -241,7 +252,8 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
         const h16x2 s2 = {sh, sh};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const h16x8 bf = __builtin_bit_cast(h16x8, unpermute8(dequant8(wq[j], z, s2, magic)));
+            const u32x4 dq = dequant8(wq[j], z, s2, magic);
+            const h16x8 bf = __builtin_bit_cast(h16x8, APERM ? dq : unpermute8(dq));
             const int chunk = j + 4 * lhalf;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -327,7 +339,8 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
                     float g = acc[i][j];
                     g *= 1.0f / (1.0f + expf(-g));
                     const float v = g * xch[((wave >> 1) * 64 + i * 16 + j) * 64 + lane];
-                    p.out[0][(size_t)p.out_off[0] + (size_t)m * p.ldo[0] + wb.row0 + col] = float_to_half_bits(v);
+                    const int n = wb.row0 + col;
+                    p.out[0][(size_t)p.out_off[0] + (size_t)m * p.ldo[0] + (p.out_perm ? permuted_index(n) : n)] = float_to_half_bits(v);
                 }
             }
         }
@@ -403,7 +416,8 @@ __global__ __launch_bounds__(256) void embed_rows_kernel(uint16_t* x, const uint
 // o[m] = half(x[m] * (rsqrt(mean(x[m]^2) + 1e-5) * w))  (gpu_kernels.h:72-105, one workgroup per token row).
 // 16-byte pieces; up to 4 per thread stay in registers between the two passes (rows of up to 8192), longer rows
 // re-read the rest.
-__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(uint16_t* o, const uint16_t* x, const uint16_t* weight, int size) {
+// perm: every 8 outputs are stored in the order (0,4,1,5,2,6,3,7) (what a permuted-A GEMM reads).
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(uint16_t* o, const uint16_t* x, const uint16_t* weight, int size, int perm) {
     __shared__ float red[4];
     constexpr int NP = 4;
     const int tid = threadIdx.x;
@@ -427,7 +441,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(uint16_t* o, const ui
         }
         return part;
     };
-    auto scale = [](const u32x4 p, const u32x4 wv, float ss) {
+    auto scale = [perm](const u32x4 p, const u32x4 wv, float ss) {
         u32x4 r;
 #pragma unroll
         for (int k = 0; k < 4; k++) {
@@ -437,7 +451,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(uint16_t* o, const ui
             q[1] = (h16_t)((float)h[1] * (ss * (float)hw[1]));
             r[k] = as_u32(q);
         }
-        return r;
+        return perm ? permute8(r) : r;
     };
     float part = 0.0f;
 #pragma unroll
@@ -498,7 +512,7 @@ constexpr int BQ = 16;
 template <int LP>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(uint16_t* out, const uint16_t* q, const uint16_t* key_cache,
                                                            const uint16_t* value_cache, int num_heads, int head_size, int kv_mul,
-                                                           int M, int pos0) {
+                                                           int M, int pos0, int out_perm) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int h = blockIdx.y;
     const int mq0 = blockIdx.x * BQ;
@@ -576,9 +590,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(uint16_t* out, const 
         for (int a = 0; a < 4; a++) {
             const int qi = qg * 4 + a;
             if (qi < nq) {
-                uint16_t* o = out + ((size_t)(mq0 + qi) * num_heads + h) * head_size + np * 2;
-                o[0] = float_to_half_bits(acc[a][0]);
-                o[1] = float_to_half_bits(acc[a][1]);
+                uint16_t* o = out + ((size_t)(mq0 + qi) * num_heads + h) * head_size;
+                o[out_perm ? permuted_index(np * 2) : np * 2] = float_to_half_bits(acc[a][0]);
+                o[out_perm ? permuted_index(np * 2 + 1) : np * 2 + 1] = float_to_half_bits(acc[a][1]);
             }
         }
     }
@@ -597,7 +611,7 @@ constexpr int VT_STRIDE = 72; // halves per row of the transposed value tile (64
 
 __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, const uint16_t* q, const uint16_t* key_cache,
                                                                 const uint16_t* value_cache, int num_heads, int kv_mul, int M,
-                                                                int pos0, int s_stride) {
+                                                                int pos0, int s_stride, int out_perm) {
     constexpr int HS = 128;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     uint16_t* S = reinterpret_cast<uint16_t*>(smem);                          // [AQ][s_stride]
@@ -747,7 +761,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, c
 #pragma unroll
     for (int j = 0; j < 16; j++) {
         const int row = (j >> 2) * 8 + lh * 4 + (j & 3);
-        if (row < nq) out[((size_t)(mq0 + row) * num_heads + h) * HS + wave * 32 + l32] = float_to_half_bits(oacc[j]);
+        const int d = wave * 32 + l32;
+        if (row < nq) out[((size_t)(mq0 + row) * num_heads + h) * HS + (out_perm ? permuted_index(d) : d)] = float_to_half_bits(oacc[j]);
     }
 }
 
@@ -795,8 +810,11 @@ int awq_gemm_device_setup(int device) {
     }
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (!g_gemm_lds_raised[device]) {
-        hipError_t e = hipFuncSetAttribute((const void*)pf::gemm_int4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipError_t e = hipFuncSetAttribute((const void*)pf::gemm_int4_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                            pf::GEMM_LDS_BYTES);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void*)pf::gemm_int4_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    pf::GEMM_LDS_BYTES);
         if (e != hipSuccess) {
             awq_set_error("hipFuncSetAttribute(gemm_int4) failed: %s", hipGetErrorString(e));
             return AWQ_ERR_HIP;
@@ -817,7 +835,8 @@ int awq_gemm_device_setup(int device) {
 
 // ---------------------------------------------------------------- launchers (internal)
 // static_ws: take the split-K workspace from the file-scope device array (no allocation) instead of the context's.
-static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* what, bool static_ws = false) {
+// a_perm: A holds every 8 activations in the order (0,4,1,5,2,6,3,7).
+static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* what, bool a_perm, bool static_ws = false) {
     // the kernel's 80 KB of LDS exceed the default dynamic limit; raised per device when a context is created
     // (contexts on a caller's stream included), here only for a device that was missed
     if (ctx->device < 0 || ctx->device >= kMaxDevices || !g_gemm_lds_raised[ctx->device]) {
@@ -875,7 +894,10 @@ static int launch_gemm(awq_ctx* ctx, pf::GemmParams& p, int ntiles, const char* 
     }
     // ids go round-robin over the 8 XCDs; each XCD takes every 8th weight tile with all of its M tiles (and K halves)
     const int grid = 8 * p.mtiles * p.ksplit * div_up(ntiles, 8);
-    hipLaunchKernelGGL(pf::gemm_int4_kernel, dim3(grid), dim3(256), pf::GEMM_LDS_BYTES, ctx->stream, p);
+    if (a_perm)
+        hipLaunchKernelGGL(pf::gemm_int4_kernel<true>, dim3(grid), dim3(256), pf::GEMM_LDS_BYTES, ctx->stream, p);
+    else
+        hipLaunchKernelGGL(pf::gemm_int4_kernel<false>, dim3(grid), dim3(256), pf::GEMM_LDS_BYTES, ctx->stream, p);
     return awq_check_launch(what);
 }
 
@@ -902,16 +924,16 @@ static void gemm_common(pf::GemmParams& p, const uint16_t* A, int lda, int M, in
 }
 
 int awq_launch_gemm_single(awq_ctx* ctx, uint16_t* out, long long ldo, const uint16_t* A, int lda, int M, const awq_qweight* w,
-                           int K, int N, int accum, bool static_ws) {
+                           int K, int N, int accum, bool static_ws, bool a_perm) {
     pf::GemmParams p;
     gemm_common(p, A, lda, M, K, accum ? pf::EPI_RESID : pf::EPI_STORE);
     set_mat(p, 0, w, N, out, ldo, 0);
-    return launch_gemm(ctx, p, N / pf::BN, "gemm_int4", static_ws);
+    return launch_gemm(ctx, p, N / pf::BN, "gemm_int4", a_perm, static_ws);
 }
 
 int awq_launch_gemm_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, long long kv_row0_off,
                         const uint16_t* A, int lda, int M, const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw,
-                        int K, int Nq, int Nkv, const float2* rope128, int pos0) {
+                        int K, int Nq, int Nkv, const float2* rope128, int pos0, bool a_perm) {
     pf::GemmParams p;
     gemm_common(p, A, lda, M, K, pf::EPI_QKV);
     p.rope = rope128;  // non-null only with 128-wide heads
@@ -919,16 +941,17 @@ int awq_launch_gemm_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t
     set_mat(p, 0, qw, Nq, q, Nq, 0);
     set_mat(p, 1, kw, Nkv, key_cache, Nkv, kv_row0_off);
     set_mat(p, 2, vw, Nkv, value_cache, Nkv, kv_row0_off);
-    return launch_gemm(ctx, p, (Nq + 2 * Nkv) / pf::BN, "gemm_int4_qkv");
+    return launch_gemm(ctx, p, (Nq + 2 * Nkv) / pf::BN, "gemm_int4_qkv", a_perm);
 }
 
 int awq_launch_gemm_ffn(awq_ctx* ctx, uint16_t* hb, const uint16_t* A, int lda, int M, const awq_qweight* gate_w,
-                        const awq_qweight* up_w, int K, int N) {
+                        const awq_qweight* up_w, int K, int N, bool a_perm, bool out_perm) {
     pf::GemmParams p;
     gemm_common(p, A, lda, M, K, pf::EPI_FFN);
+    p.out_perm = out_perm;
     set_mat(p, 0, gate_w, N, hb, N, 0);
     set_mat(p, 1, up_w, N, hb, N, 0);
-    return launch_gemm(ctx, p, N / 64, "gemm_int4_ffn");
+    return launch_gemm(ctx, p, N / 64, "gemm_int4_ffn", a_perm);
 }
 
 int awq_launch_embed_rows(awq_ctx* ctx, uint16_t* x, const uint16_t* table, int dim, const int* tokens, int pos0, int M) {
@@ -936,8 +959,8 @@ int awq_launch_embed_rows(awq_ctx* ctx, uint16_t* x, const uint16_t* table, int 
     return awq_check_launch("embed_rows");
 }
 
-int awq_launch_rmsnorm_rows(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const uint16_t* w, int size, int M) {
-    hipLaunchKernelGGL(pf::rmsnorm_rows_kernel, dim3(M), dim3(256), 0, ctx->stream, o, x, w, size);
+int awq_launch_rmsnorm_rows(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const uint16_t* w, int size, int M, int perm) {
+    hipLaunchKernelGGL(pf::rmsnorm_rows_kernel, dim3(M), dim3(256), 0, ctx->stream, o, x, w, size, perm);
     return awq_check_launch("rmsnorm_rows");
 }
 
@@ -956,7 +979,7 @@ int awq_prefill_attention_max_positions(int head_size) {
 }
 
 int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, const uint16_t* kc, const uint16_t* vc, int nh, int hs,
-                            int kv_mul, int M, int pos0) {
+                            int kv_mul, int M, int pos0, int out_perm) {
     if (hs == 128) {
         const int s_stride = ((pos0 + M + 63) & ~63) + 8;
         const size_t lds = (size_t)pf::AQ * s_stride * 2 + 2 * 128 * pf::VT_STRIDE * 2;
@@ -973,7 +996,7 @@ int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, cons
             }
         }
         hipLaunchKernelGGL(pf::attn_prefill_mfma_kernel, dim3(div_up(M, pf::AQ), nh), dim3(256), lds, ctx->stream, out, q, kc, vc,
-                           nh, kv_mul, M, pos0, s_stride);
+                           nh, kv_mul, M, pos0, s_stride, out_perm);
         return awq_check_launch("attn_prefill_mfma");
     }
     const int nk_max = (pos0 + M + 7) & ~7;
@@ -994,7 +1017,7 @@ int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, cons
             }                                                                                                             \
         }                                                                                                                 \
         hipLaunchKernelGGL((pf::attn_prefill_kernel<LPV>), grid, dim3(256), lds, ctx->stream, out, q, kc, vc, nh, hs, kv_mul, \
-                           M, pos0);                                                                                      \
+                           M, pos0, out_perm);                                                                            \
     } while (0)
     switch (hs) {
         case 64: AWQ_ATTN_PF(8); break;
@@ -1026,7 +1049,7 @@ int awq_gemm_int4(awq_ctx* ctx, uint16_t* out, int ldo, const uint16_t* a, int l
         awq_set_error("awq_gemm_int4: needs M > 0, K %% 32 == 0, N %% 128 == 0, lda %% 8 == 0 (got M=%d K=%d N=%d lda=%d)", M, K, N, lda);
         return AWQ_ERR_SHAPE;
     }
-    return awq_launch_gemm_single(ctx, out, ldo, a, lda, M, w, K, N, accum, false);
+    return awq_launch_gemm_single(ctx, out, ldo, a, lda, M, w, K, N, accum, false, false);
 }
 
 int awq_gemm_int4_static(awq_ctx* ctx, uint16_t* out, int ldo, const uint16_t* a, int lda, int M, const awq_qweight* w, int K,
@@ -1040,7 +1063,7 @@ int awq_gemm_int4_static(awq_ctx* ctx, uint16_t* out, int ldo, const uint16_t* a
     }
     AWQ_REQUIRE(ctx->device >= 0 && ctx->device < kMaxDevices && g_scratch_ptr[ctx->device] && g_gemm_lds_raised[ctx->device],
                 AWQ_ERR_HIP, "the static workspace was not set up on this device when the context was created");
-    return awq_launch_gemm_single(ctx, out, ldo, a, lda, M, w, K, N, accum, true);
+    return awq_launch_gemm_single(ctx, out, ldo, a, lda, M, w, K, N, accum, true, false);
 }
 
 }  // extern "C"

@@ -35,18 +35,18 @@ int awq_sampler_run(awq_sampler* s, uint16_t* logits, int* tokens, volatile int*
                     int* mirror);
 // prefill.hip
 int awq_launch_gemm_single(awq_ctx* ctx, uint16_t* out, long long ldo, const uint16_t* A, int lda, int M, const awq_qweight* w,
-                           int K, int N, int accum, bool static_ws);
+                           int K, int N, int accum, bool static_ws, bool a_perm);
 int awq_launch_gemm_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, long long kv_row0_off,
                         const uint16_t* A, int lda, int M, const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw,
-                        int K, int Nq, int Nkv, const float2* rope128, int pos0);
+                        int K, int Nq, int Nkv, const float2* rope128, int pos0, bool a_perm);
 int awq_launch_gemm_ffn(awq_ctx* ctx, uint16_t* hb, const uint16_t* A, int lda, int M, const awq_qweight* gate_w,
-                        const awq_qweight* up_w, int K, int N);
+                        const awq_qweight* up_w, int K, int N, bool a_perm, bool out_perm);
 int awq_launch_embed_rows(awq_ctx* ctx, uint16_t* x, const uint16_t* table, int dim, const int* tokens, int pos0, int M);
-int awq_launch_rmsnorm_rows(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const uint16_t* w, int size, int M);
+int awq_launch_rmsnorm_rows(awq_ctx* ctx, uint16_t* o, const uint16_t* x, const uint16_t* w, int size, int M, int perm);
 int awq_launch_rope_rows(awq_ctx* ctx, uint16_t* q, uint16_t* kcache_layer, int nh, int nkv, int hs, int pos0, float theta, int M,
                          const float2* table);
 int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, const uint16_t* kc, const uint16_t* vc, int nh, int hs,
-                            int kv_mul, int M, int pos0);
+                            int kv_mul, int M, int pos0, int out_perm);
 int awq_launch_set_pos(awq_ctx* ctx, int* pos_dev, volatile int* pos_host, int value);
 int awq_prefill_attention_max_positions(int head_size);
 int awq_launch_copy_row(awq_ctx* ctx, uint16_t* dst, const uint16_t* src, int n);
@@ -851,25 +851,28 @@ int awq_transformer_prefill(awq_transformer* t, int n_tokens, int gen_token) {
         const int M = (n_batched - done < t->pf_rows) ? n_batched - done : t->pf_rows;
         const int pos0 = pos_start + done;
         if ((r = awq_launch_embed_rows(ctx, t->pf_x, t->embed, dim, t->tokens_dev, pos0, M))) return r;
+        // The activations that feed a GEMM (xb, att, hb) are written with every 8 values in the order the packed weights
+        // dequantise in, so that the GEMMs multiply them without reordering either operand; x, q and the KV cache
+        // keep the natural order.
         for (int l = 0; l < p.n_layers; l++) {
             const awq_layer_weights& L = t->layers[l];
             const long long loff = (long long)l * p.seq_len * kv_dim;
-            if ((r = awq_launch_rmsnorm_rows(ctx, t->pf_xb, t->pf_x, L.rms_att_weight, dim, M))) return r;
+            if ((r = awq_launch_rmsnorm_rows(ctx, t->pf_xb, t->pf_x, L.rms_att_weight, dim, M, 1))) return r;
             // 128-wide heads: the QKV GEMM rotates q and k in its epilogue; other head sizes run the RoPE kernel
             const float2* rope128 = (hs == 128) ? t->rope_table : nullptr;
             if ((r = awq_launch_gemm_qkv(ctx, t->pf_q, t->s.key_cache, t->s.value_cache, loff + (long long)pos0 * kv_dim, t->pf_xb,
-                                         dim, M, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, kv_dim, rope128, pos0)))
+                                         dim, M, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, kv_dim, rope128, pos0, true)))
                 return r;
             if (!rope128 && (r = awq_launch_rope_rows(ctx, t->pf_q, t->s.key_cache + loff, p.n_heads, p.n_kv_heads, hs, pos0,
                                                       p.rope_theta, M, t->rope_table)))
                 return r;
             if ((r = awq_launch_attn_prefill(ctx, t->pf_att, t->pf_q, t->s.key_cache + loff, t->s.value_cache + loff, p.n_heads, hs,
-                                             kv_mul, M, pos0)))
+                                             kv_mul, M, pos0, 1)))
                 return r;
-            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_att, dim, M, &L.wq_o, dim, dim, 1, false))) return r;
-            if ((r = awq_launch_rmsnorm_rows(ctx, t->pf_xb, t->pf_x, L.rms_ffn_weight, dim, M))) return r;
-            if ((r = awq_launch_gemm_ffn(ctx, t->pf_hb, t->pf_xb, dim, M, &L.wq_gate, &L.wq_up, dim, hidden))) return r;
-            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_hb, hidden, M, &L.wq_down, hidden, dim, 1, false))) return r;
+            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_att, dim, M, &L.wq_o, dim, dim, 1, false, true))) return r;
+            if ((r = awq_launch_rmsnorm_rows(ctx, t->pf_xb, t->pf_x, L.rms_ffn_weight, dim, M, 1))) return r;
+            if ((r = awq_launch_gemm_ffn(ctx, t->pf_hb, t->pf_xb, dim, M, &L.wq_gate, &L.wq_up, dim, hidden, true, true))) return r;
+            if ((r = awq_launch_gemm_single(ctx, t->pf_x, dim, t->pf_hb, hidden, M, &L.wq_down, hidden, dim, 1, false, true))) return r;
         }
         if (done + M == n_tokens) {
             // last token: final norm, classifier and the greedy sampler exactly as the decode path does them
