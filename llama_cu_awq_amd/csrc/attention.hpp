@@ -36,18 +36,21 @@ __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att
     const bool mine = NS == 1 || j / (LP / NS) == slice;  // this lane's 8 value dimensions belong to the slice
     // The value rows of the first round are requested together with its key rows: at short context that is all of
     // them, and the softmax then runs while they are on their way.
+    // Every load below is unconditional: positions past the end are clamped to the last one, and lanes whose value
+    // dimensions belong to another slice re-read the query instead (one line for the whole wave).  A load inside a
+    // branch makes the compiler wait for it before it issues the next one, which serialises the memory round trips.
     u32x4 vfirst[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-        const int t = tfirst + k * tstep;
-        if (t < size && mine) vfirst[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+        const int t = min(tfirst + k * tstep, size - 1);
+        vfirst[k] = *reinterpret_cast<const u32x4*>(mine ? vh + (size_t)t * row_stride : q_head);
     }
     for (int t0 = tfirst; t0 - tfirst < size; t0 += 4 * tstep) {
         u32x4 kv[4];
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            const int t = t0 + k * tstep;
-            if (t < size) kv[k] = *reinterpret_cast<const u32x4*>(kh + (size_t)t * row_stride);
+            const int t = min(t0 + k * tstep, size - 1);
+            kv[k] = *reinterpret_cast<const u32x4*>(kh + (size_t)t * row_stride);
         }
 #pragma unroll
         for (int k = 0; k < 4; k++) {
@@ -86,8 +89,8 @@ __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att
             const int t = t0 + k * tstep;
             if (t0 == tfirst)
                 vv[k] = vfirst[k];
-            else if (t < size && mine)
-                vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
+            else
+                vv[k] = *reinterpret_cast<const u32x4*>(mine ? vh + (size_t)min(t, size - 1) * row_stride : q_head);
         }
 #pragma unroll
         for (int k = 0; k < 4; k++) {

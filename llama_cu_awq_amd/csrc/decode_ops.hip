@@ -99,8 +99,9 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(uint16_t* att, const u
     u32x4 kv[ITERS];
 #pragma unroll
     for (int it = 0; it < ITERS; it++) {
-        const int t = t0 + wave * 16 + it * PW + pr;
-        if (t < size) kv[it] = *reinterpret_cast<const u32x4*>(kh + (size_t)t * row_stride);
+        // (clamped, not skipped: a load inside a branch makes the compiler wait for it before the next one)
+        const int t = min(t0 + wave * 16 + it * PW + pr, size - 1);
+        kv[it] = *reinterpret_cast<const u32x4*>(kh + (size_t)t * row_stride);
     }
 #pragma unroll
     for (int it = 0; it < ITERS; it++) {
@@ -138,16 +139,13 @@ __global__ __launch_bounds__(1024) void attn_pv_sliced_kernel(uint16_t* output, 
     u32x4 vv[R];
     uint16_t sv[R];
     auto request = [&](int t0) {
+        // positions past the end are clamped, not skipped: a load inside a branch makes the compiler wait for it
+        // before it issues the next one
 #pragma unroll
-        for (int k = 0; k < R; k++) {
-            const int t = t0 + pg + NG * k;
-            if (t < size) sv[k] = a[t];
-        }
+        for (int k = 0; k < R; k++) sv[k] = a[min(t0 + pg + NG * k, size - 1)];
 #pragma unroll
-        for (int k = 0; k < R; k++) {
-            const int t = t0 + pg + NG * k;
-            if (t < size) vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
-        }
+        for (int k = 0; k < R; k++)
+            vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)min(t0 + pg + NG * k, size - 1) * row_stride);
     };
     request(0);
     // statistics over all positions (gpu_kernels.h:376-400; the max seed is the reference's idle-lane 0 when its
@@ -262,20 +260,16 @@ __global__ __launch_bounds__(1024) void attn_pv_partial_kernel(float* part, cons
     // Loads return in order: the scores that the statistics need (two per thread cover 2048 positions) are requested
     // ahead of the value rows, so that the statistics are computed while the rows are still on their way.
     uint16_t stat[2];
+    // (positions past the end are clamped, not skipped: a load inside a branch makes the compiler wait for it before
+    // it issues the next one)
 #pragma unroll
-    for (int j = 0; j < 2; j++)
-        if (tid + 1024 * j < size) stat[j] = a[tid + 1024 * j];
+    for (int j = 0; j < 2; j++) stat[j] = a[min(tid + 1024 * j, size - 1)];
     auto request = [&](int t0) {
 #pragma unroll
-        for (int k = 0; k < R; k++) {
-            const int t = t0 + rg + 128 * k;
-            if (t < t_end) sv[k] = a[t];
-        }
+        for (int k = 0; k < R; k++) sv[k] = a[min(t0 + rg + 128 * k, size - 1)];
 #pragma unroll
-        for (int k = 0; k < R; k++) {
-            const int t = t0 + rg + 128 * k;
-            if (t < t_end) vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)t * row_stride);
-        }
+        for (int k = 0; k < R; k++)
+            vv[k] = *reinterpret_cast<const u32x4*>(vh + (size_t)min(t0 + rg + 128 * k, size - 1) * row_stride);
     };
     request(t_begin);
     // statistics over all positions (the max seed is the reference's idle-lane 0 when its 1024-thread block is not full)
