@@ -247,6 +247,7 @@ __global__ __launch_bounds__(1024) void attn_pv_partial_kernel(float* part, cons
     constexpr int R = kPvPartialRows;
     __shared__ float red[16];
     __shared__ float acc_lds[16][64];
+    __shared__ float pl[8 * 136];  // probabilities of the positions in flight: [row of the group][row group], padded
     const int size = *pPos + 1;
     const int h = blockIdx.x, chunk = blockIdx.y, slice = blockIdx.z;
     const int per = (size + chunks - 1) / chunks;
@@ -306,14 +307,27 @@ __global__ __launch_bounds__(1024) void attn_pv_partial_kernel(float* part, cons
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.0f;
+    static_assert(R == 8, "lane ql of a row group computes the probability of the group's row ql");
     for (int t0 = t_begin; t0 < t_end; t0 += 128 * R) {
-        if (t0 != t_begin) request(t0);
+        if (t0 != t_begin) {
+            __syncthreads();  // the previous round's probabilities have been read
+            request(t0);
+        }
+        // The 8 lanes of a row group need the same 8 probabilities: lane ql computes the one of row ql (exponential
+        // and correctly rounded quotient once per position instead of 8 times) and the group shares them through LDS.
+        {
+            uint16_t sq = sv[0];
+#pragma unroll
+            for (int k = 1; k < R; k++) sq = ql == k ? sv[k] : sq;
+            const float e = expf(half_bits_to_float(sq) - m);
+            pl[ql * 136 + rg] = half_bits_to_float(float_to_half_bits(e / sum));  // probability rounded to fp16
+        }
+        __syncthreads();
 #pragma unroll
         for (int k = 0; k < R; k++) {
             const int t = t0 + rg + 128 * k;
             if (t < t_end) {
-                const float e = expf(half_bits_to_float(sv[k]) - m);
-                const float p = half_bits_to_float(float_to_half_bits(e / sum));  // probability rounded to fp16
+                const float p = pl[k * 136 + rg];
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const h16x2 hv = as_h2(vv[k][i]);
