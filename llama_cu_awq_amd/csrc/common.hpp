@@ -115,6 +115,17 @@ __device__ __forceinline__ uint32_t as_u32(h16x2 h) { return __builtin_bit_cast(
 __device__ __forceinline__ float half_bits_to_float(uint16_t b) { return (float)__builtin_bit_cast(h16_t, b); }
 __device__ __forceinline__ uint16_t float_to_half_bits(float f) { return __builtin_bit_cast(uint16_t, (h16_t)f); }  // RNE
 
+// RoPE rotation of one pair, (v0, v1) -> (v0 c - v1 s, v0 s + v1 c) (gpu_kernels.h:355-361).  One fixed evaluation for
+// every kernel that rotates (second product rounded on its own, first product fused with the sum), so that the
+// separate kernel, the matrix-vector epilogue, the batched GEMM epilogue and the per-token kernel agree bit for bit
+// whatever the compiler would have contracted in each of them.
+__device__ __forceinline__ void rope_rotate(float v0, float v1, float c, float s, float& o0, float& o1) {
+#pragma clang fp contract(off)
+    const float t0 = v1 * s, t1 = v1 * c;
+    o0 = __builtin_fmaf(v0, c, -t0);
+    o1 = __builtin_fmaf(v0, s, t1);
+}
+
 // Streaming (non-temporal) loads for data that is read exactly once.
 __device__ __forceinline__ u32x4 load_nt(const u32x4* p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ uint32_t load_nt(const uint32_t* p) { return __builtin_nontemporal_load(p); }

@@ -64,14 +64,17 @@ __global__ void rope_kernel(uint16_t* sq, uint16_t* sk_base, int num_kv_heads, i
     uint16_t* q = sq + (size_t)h * head_size;
     const float q0 = half_bits_to_float(q[i]);
     const float q1 = half_bits_to_float(q[i + half_size]);
-    q[i] = float_to_half_bits(q0 * fcr - q1 * fci);
-    q[i + half_size] = float_to_half_bits(q0 * fci + q1 * fcr);
+    float r0, r1;
+    rope_rotate(q0, q1, fcr, fci, r0, r1);
+    q[i] = float_to_half_bits(r0);
+    q[i + half_size] = float_to_half_bits(r1);
     if (h < num_kv_heads) {
         uint16_t* k = sk_base + (size_t)loff + (size_t)pos * num_kv_heads * head_size + (size_t)h * head_size;
         const float k0 = half_bits_to_float(k[i]);
         const float k1 = half_bits_to_float(k[i + half_size]);
-        k[i] = float_to_half_bits(k0 * fcr - k1 * fci);
-        k[i + half_size] = float_to_half_bits(k0 * fci + k1 * fcr);
+        rope_rotate(k0, k1, fcr, fci, r0, r1);
+        k[i] = float_to_half_bits(r0);
+        k[i + half_size] = float_to_half_bits(r1);
     }
 }
 

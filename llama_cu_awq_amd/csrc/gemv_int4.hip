@@ -169,8 +169,10 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
                         const float v0 = half_bits_to_float(float_to_half_bits(sum[r]));
                         const float v1 = half_bits_to_float(float_to_half_bits(sum[r + 1]));
                         const float2 c = cs_tab[row % half];
-                        out[row] = float_to_half_bits(v0 * c.x - v1 * c.y);
-                        out[row + half] = float_to_half_bits(v0 * c.y + v1 * c.x);
+                        float r0, r1;
+                        rope_rotate(v0, v1, c.x, c.y, r0, r1);
+                        out[row] = float_to_half_bits(r0);
+                        out[row + half] = float_to_half_bits(r1);
                     }
                 }
             } else {

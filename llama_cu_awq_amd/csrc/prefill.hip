@@ -18,6 +18,7 @@
 
 typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace pf {
 
@@ -314,93 +315,121 @@ __global__ __launch_bounds__(256, 2) void gemm_int4_kernel(const GemmParams p) {
             for (int j = 0; j < 16; j++) acc[i][j] += other[((wave * 4 + i) * 16 + j) * 64 + lane];
     }
 
-    // epilogue: acc[i][j] is D[row = 32*i + 8*(j/4) + 4*(lane/32) + j%4][col = lane%32] of the wave's 32 columns
-    const int col = lane & 31;
-    if (p.epi == EPI_FFN) {
-        // waves 0, 2 hold gate columns, waves 1, 3 the up columns of the same row indices: the up waves pass their
-        // accumulators through LDS once the loads still in flight have landed there
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        float* xch = reinterpret_cast<float*>(lds_bytes);  // [2 pairs][64 values][64 lanes]
-        if (wave & 1) {
+    // ---- epilogue.  acc[i][j] is D[row = 32*i + 8*(j/4) + 4*(lane/32) + j%4][col = lane%32] of the wave's 32 columns:
+    // a lane holds one column, so stored from registers every value would be a 2-byte access of its own (measured: 15 us
+    // for the RoPE form, 12 for SiLU, 5 for the residual form, of a 50 us K loop).  The four waves therefore pass their
+    // accumulators through the now idle LDS rings as one fp32 tile [wave][128 rows][32 columns], and every lane then
+    // owns 8 consecutive columns of a row: one 16-byte store (and one 16-byte load of the old values, the rotation
+    // factors or the partner columns) per 8 results.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no direct-to-LDS load is still on its way
+    __syncthreads();
+    float* tile_f = reinterpret_cast<float*>(lds_bytes);
+    {
+        float* mine = tile_f + wave * 4096 + (lane >> 5) * 128 + (lane & 31);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+        for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int j = 0; j < 16; j++) xch[((wave >> 1) * 64 + i * 16 + j) * 64 + lane] = acc[i][j];
+            for (int j = 0; j < 16; j++) mine[(i * 32 + (j >> 2) * 8 + (j & 3)) * 32] = acc[i][j];
+    }
+    __syncthreads();
+    const int chunk = lane & 3, rsub = lane >> 2;  // 8 columns of row rsub, rsub + 16, ...
+    auto read8 = [&](int w, int row, float (&v)[8]) {
+        const f32x4* src = reinterpret_cast<const f32x4*>(tile_f + w * 4096 + row * 32 + chunk * 8);
+        const f32x4 a = src[0], b = src[1];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            v[e] = a[e];
+            v[4 + e] = b[e];
         }
-        __syncthreads();
-        if (!(wave & 1)) {
+    };
+    auto pack8 = [](const float (&v)[8]) {
+        u32x4 o;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+        for (int e = 0; e < 4; e++) o[e] = (uint32_t)float_to_half_bits(v[2 * e]) | ((uint32_t)float_to_half_bits(v[2 * e + 1]) << 16);
+        return o;
+    };
+    if (p.epi == EPI_FFN) {
+        // waves 0, 2 hold gate columns, waves 1, 3 the up columns of the same weight rows: the two waves of a pair take
+        // 64 tile rows each
+        const int wg = wave & ~1;
+        const int n0 = block_map(p, tile, wg).row0 + chunk * 8;
+        uint16_t* o = p.out[0] + (size_t)p.out_off[0] + n0;
 #pragma unroll
-                for (int j = 0; j < 16; j++) {
-                    const int m = m0 + i * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
-                    if (m >= p.M) continue;
-                    float g = acc[i][j];
-                    g *= 1.0f / (1.0f + expf(-g));
-                    const float v = g * xch[((wave >> 1) * 64 + i * 16 + j) * 64 + lane];
-                    const int n = wb.row0 + col;
-                    p.out[0][(size_t)p.out_off[0] + (size_t)m * p.ldo[0] + (p.out_perm ? permuted_index(n) : n)] = float_to_half_bits(v);
-                }
+        for (int it = 0; it < 4; it++) {
+            const int row = (wave & 1) * 64 + it * 16 + rsub;
+            const int m = m0 + row;
+            float g[8], u[8], v[8];
+            read8(wg, row, g);
+            read8(wg + 1, row, u);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float s = g[e] * (1.0f / (1.0f + expf(-g[e])));
+                v[e] = s * u[e];
             }
+            if (p.out_perm) {  // (0,4,1,5,2,6,3,7): the order a permuted-A GEMM reads
+                const float t[8] = {v[0], v[4], v[1], v[5], v[2], v[6], v[3], v[7]};
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] = t[e];
+            }
+            if (m < p.M) *reinterpret_cast<u32x4*>(o + (size_t)m * p.ldo[0]) = pack8(v);
         }
         return;
     }
     const int mat = wb.mat;
+    uint16_t* o = (mat == 0 ? p.out[0] : (mat == 1 ? p.out[1] : p.out[2])) +
+                  (size_t)(mat == 0 ? p.out_off[0] : (mat == 1 ? p.out_off[1] : p.out_off[2])) + wb.row0 + chunk * 8;
+    const size_t ld = (size_t)(mat == 0 ? p.ldo[0] : (mat == 1 ? p.ldo[1] : p.ldo[2]));
     if (p.rope && mat < 2) {
-        // The tile is one head: column c < 64 rotates with column c + 64, which the wave two further on holds in the
-        // same lane and accumulator element.  Values are rounded to fp16 first and rotated in fp32, as the separate
-        // kernel does on the stored q and k (gpu_kernels.h:351-361); the exchange goes through the idle LDS rings.
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        float* xch = reinterpret_cast<float*>(lds_bytes);  // [4 waves][64 values][64 lanes]
+        // The tile is one head: column c < 64 rotates with column c + 64, which the wave two further on holds.  Values
+        // are rounded to fp16 first and rotated in fp32, as the separate kernel does on the stored q and k
+        // (gpu_kernels.h:351-361).  (cos, sin) of 8 consecutive pairs are 64 contiguous bytes of the table.
+        const int pair0 = (wave & 1) * 32 + chunk * 8;  // 0 .. 63
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int it = 0; it < 8; it++) {
+            const int row = it * 16 + rsub;
+            const int m = m0 + row;
+            const f32x4* cs = reinterpret_cast<const f32x4*>(p.rope + (size_t)(p.rope_pos0 + min(m, p.M - 1)) * 64 + pair0);
+            const f32x4 c0 = cs[0], c1 = cs[1], c2 = cs[2], c3 = cs[3];
+            const float cosv[8] = {c0[0], c0[2], c1[0], c1[2], c2[0], c2[2], c3[0], c3[2]};
+            const float sinv[8] = {c0[1], c0[3], c1[1], c1[3], c2[1], c2[3], c3[1], c3[3]};
+            float a[8], b[8], v[8];
+            read8(wave, row, a);
+            read8(wave ^ 2, row, b);
 #pragma unroll
-            for (int j = 0; j < 16; j++) {
-                acc[i][j] = half_bits_to_float(float_to_half_bits(acc[i][j]));
-                xch[(wave * 64 + i * 16 + j) * 64 + lane] = acc[i][j];
+            for (int e = 0; e < 8; e++) {
+                const float own = half_bits_to_float(float_to_half_bits(a[e]));
+                const float other = half_bits_to_float(float_to_half_bits(b[e]));
+                // columns below 64 are the first elements of their pairs, the others the second
+                float r0, r1;
+                if (wave < 2) rope_rotate(own, other, cosv[e], sinv[e], r0, r1);
+                else rope_rotate(other, own, cosv[e], sinv[e], r0, r1);
+                v[e] = wave < 2 ? r0 : r1;
             }
-        __syncthreads();
-        uint16_t* ro = (mat == 0 ? p.out[0] : p.out[1]) + (size_t)(mat == 0 ? p.out_off[0] : p.out_off[1]) + wb.row0 + col;
-        const size_t rld = (size_t)(mat == 0 ? p.ldo[0] : p.ldo[1]);
-        const int pair = (wave & 1) * 32 + col;  // 0 .. 63
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-#pragma unroll
-            for (int j = 0; j < 16; j++) {
-                const int m = m0 + i * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
-                if (m >= p.M) continue;
-                const float2 cs = p.rope[(size_t)(p.rope_pos0 + m) * 64 + pair];
-                const float other = xch[((wave ^ 2) * 64 + i * 16 + j) * 64 + lane];
-                const float v = wave < 2 ? acc[i][j] * cs.x - other * cs.y : other * cs.y + acc[i][j] * cs.x;
-                ro[(size_t)m * rld] = float_to_half_bits(v);
-            }
+            if (m < p.M) *reinterpret_cast<u32x4*>(o + (size_t)m * ld) = pack8(v);
         }
         return;
     }
-    uint16_t* o = (mat == 0 ? p.out[0] : (mat == 1 ? p.out[1] : p.out[2])) +
-                  (size_t)(mat == 0 ? p.out_off[0] : (mat == 1 ? p.out_off[1] : p.out_off[2])) + wb.row0 + col;
-    const size_t ld = (size_t)(mat == 0 ? p.ldo[0] : (mat == 1 ? p.ldo[1] : p.ldo[2]));
+    // plain and residual forms; the old values of all 8 row passes are requested before the first is used
+    u32x4 old[8];
+    if (p.epi == EPI_RESID) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        // residual form: all 16 old values are requested before the first is used
-        uint16_t old[16];
+        for (int it = 0; it < 8; it++)
+            old[it] = *reinterpret_cast<const u32x4*>(o + (size_t)min(m0 + it * 16 + rsub, p.M - 1) * ld);
+    }
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+        const int row = it * 16 + rsub;
+        const int m = m0 + row;
+        float v[8];
+        read8(wave, row, v);
         if (p.epi == EPI_RESID) {
 #pragma unroll
-            for (int j = 0; j < 16; j++) {
-                const int m = m0 + i * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
-                old[j] = o[(size_t)min(m, p.M - 1) * ld];
+            for (int e = 0; e < 4; e++) {
+                v[2 * e] += half_bits_to_float((uint16_t)(old[it][e] & 0xFFFFu));
+                v[2 * e + 1] += half_bits_to_float((uint16_t)(old[it][e] >> 16));
             }
         }
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const int m = m0 + i * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
-            if (m >= p.M) continue;
-            float v = acc[i][j];
-            if (p.epi == EPI_RESID) v += half_bits_to_float(old[j]);
-            o[(size_t)m * ld] = float_to_half_bits(v);
-        }
+        if (m < p.M) *reinterpret_cast<u32x4*>(o + (size_t)m * ld) = pack8(v);
     }
 }
 
@@ -494,14 +523,17 @@ __global__ void rope_rows_kernel(uint16_t* q, uint16_t* kcache_layer, int num_he
     uint16_t* qh = q + ((size_t)m * num_heads + h) * head_size;
     const float q0 = half_bits_to_float(qh[i]);
     const float q1 = half_bits_to_float(qh[i + half_size]);
-    qh[i] = float_to_half_bits(q0 * fcr - q1 * fci);
-    qh[i + half_size] = float_to_half_bits(q0 * fci + q1 * fcr);
+    float r0, r1;
+    rope_rotate(q0, q1, fcr, fci, r0, r1);
+    qh[i] = float_to_half_bits(r0);
+    qh[i + half_size] = float_to_half_bits(r1);
     if (h < num_kv_heads) {
         uint16_t* k = kcache_layer + ((size_t)pos * num_kv_heads + h) * head_size;
         const float k0 = half_bits_to_float(k[i]);
         const float k1 = half_bits_to_float(k[i + half_size]);
-        k[i] = float_to_half_bits(k0 * fcr - k1 * fci);
-        k[i + half_size] = float_to_half_bits(k0 * fci + k1 * fcr);
+        rope_rotate(k0, k1, fcr, fci, r0, r1);
+        k[i] = float_to_half_bits(r0);
+        k[i + half_size] = float_to_half_bits(r1);
     }
 }
 

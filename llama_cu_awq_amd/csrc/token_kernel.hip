@@ -286,8 +286,8 @@ __device__ __forceinline__ void rope_pair(float& v0, float& v1, int i, int head_
     const float val = pos * freq;
     const float fcr = cosf(val);
     const float fci = sinf(val);
-    const float a0 = v0 * fcr - v1 * fci;
-    const float a1 = v0 * fci + v1 * fcr;
+    float a0, a1;
+    rope_rotate(v0, v1, fcr, fci, a0, a1);
     v0 = a0;
     v1 = a1;
 }
