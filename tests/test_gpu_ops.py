@@ -199,6 +199,22 @@ def test_shape_guard(ctx, K, N):
         A.matmul(ctx, buf, buf, buf, K, N)
 
 
+def test_partial_sum_input_guards(ctx):
+    """The matrix-vector product that takes its input as fp32 partial sums: 1 to 4 of them, K up to 8192, the usual shape
+    rules; the split attention rejects head sizes and head counts it has no kernel for.  Nothing is launched."""
+    buf = ctx.alloc(1 << 16)
+    qw = A.QWeight(buf, buf, buf)
+    for parts, K, N in ((0, 4096, 4096), (5, 4096, 4096), (2, 8192 + 128, 4096), (2, 12, 8), (2, 4096, 4100)):
+        with pytest.raises(A.AwqError) as e:
+            A.matmul_q_parts(ctx, buf, buf, parts, qw, K, N)
+        assert e.value.code == AWQ_ERR_SHAPE, (parts, K, N)
+    pos = ctx.upload(np.array([300], dtype=np.int32))
+    for heads, head, kv_mul in ((32, 96, 1), (300, 128, 1), (32, 128, 3)):
+        with pytest.raises(A.AwqError) as e:
+            A.MultiHeadAttention_partial(ctx, buf, buf, buf, buf, buf, heads, head, kv_mul, 512, pos)
+        assert e.value.code == AWQ_ERR_SHAPE, (heads, head, kv_mul)
+
+
 @pytest.mark.parametrize("size", [4096, 5120, 6656, 8, 1000])
 def test_rmsnorm(ctx, size):
     x = synth.normal_f16(synth.stream_key(3, "x", size), size, 0.0, 2.0)
