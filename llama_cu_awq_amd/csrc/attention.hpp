@@ -92,12 +92,22 @@ __device__ __forceinline__ void attention_head(uint16_t* out_head, uint16_t* att
             else
                 vv[k] = *reinterpret_cast<const u32x4*>(mine ? vh + (size_t)min(t, size - 1) * row_stride : q_head);
         }
+        // The LP lanes of a position all need its probability.  With 16 lanes per position (one DPP row) lane k of
+        // the row computes the one of round k (exponential and correctly rounded quotient once instead of four times
+        // per lane) and the row takes it from there.
+        float p_row = 0.0f;
+        if (LP == 16) {
+            const int t = t0 + min(j, 3) * tstep;
+            if (j < 4 && t < size) p_row = half_bits_to_float(float_to_half_bits(expf(sc[t] - m) / sum));
+        }
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const int t = t0 + k * tstep;
+            float pv;
+            if (LP == 16)
+                pv = k == 0 ? dpp_mov<0x150>(p_row) : k == 1 ? dpp_mov<0x151>(p_row) : k == 2 ? dpp_mov<0x152>(p_row) : dpp_mov<0x153>(p_row);
             if (t < size && mine) {
-                const float e = expf(sc[t] - m);
-                const float pv = half_bits_to_float(float_to_half_bits(e / sum));
+                if (LP != 16) pv = half_bits_to_float(float_to_half_bits(expf(sc[t] - m) / sum));
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const h16x2 hv = as_h2(vv[k][i]);
