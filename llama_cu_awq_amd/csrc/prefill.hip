@@ -640,16 +640,37 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(uint16_t* out, const 
 //     produces head dims 32w .. 32w+31.
 constexpr int AQ = 32;        // queries per workgroup
 constexpr int VT_STRIDE = 72; // halves per row of the transposed value tile (64 keys + 8 padding)
+constexpr int KT_STRIDE = 136; // halves per row of a wave's key tile (128 dimensions + 8 padding)
+static_assert(4 * 32 * KT_STRIDE <= 2 * 128 * VT_STRIDE, "the four key tiles share the value tiles' space");
 
-__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, const uint16_t* q, const uint16_t* key_cache,
+// a / b correctly rounded, given rcp = 1 / b correctly rounded: the product a * rcp is within one unit of the quotient,
+// and one step of a - b * q (exact in the fused multiply-add) times rcp puts it right (Markstein's correction; for
+// 0 <= a <= 1 <= b no scaling is needed).  Three instructions where the division takes eleven.
+__device__ __forceinline__ float quotient(float a, float b, float rcp) {
+#pragma clang fp contract(off)
+    const float q = a * rcp;
+    const float e = __builtin_fmaf(-b, q, a);
+    return __builtin_fmaf(e, rcp, q);
+}
+
+__global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(uint16_t* out, const uint16_t* q, const uint16_t* key_cache,
                                                                 const uint16_t* value_cache, int num_heads, int kv_mul, int M,
                                                                 int pos0, int s_stride, int out_perm) {
     constexpr int HS = 128;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     uint16_t* S = reinterpret_cast<uint16_t*>(smem);                          // [AQ][s_stride]
     uint16_t* Vt = reinterpret_cast<uint16_t*>(smem + AQ * s_stride * 2);     // [2][HS][VT_STRIDE]
-    const int h = blockIdx.y;
-    const int mq0 = blockIdx.x * AQ;
+    // Workgroup ids go round-robin over the 8 XCDs: all query blocks of a head run on one XCD, so that the head's key
+    // and value rows come from memory into one L2 only (measured: with a head's blocks spread over all XCDs the score
+    // phase was bound by 8 copies of every row crossing the fabric).  A head's blocks are dealt longest first; the
+    // second half of an XCD's heads shortest first, so that the two workgroups of a compute unit tend to be one long
+    // and one short.
+    const int nqb = (M + AQ - 1) / AQ, hpx = (num_heads + 7) >> 3;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int h = xcd + 8 * (slot / nqb);
+    if (h >= num_heads) return;
+    const int qb = (slot / nqb) * 2 >= hpx ? slot % nqb : nqb - 1 - slot % nqb;
+    const int mq0 = qb * AQ;
     const int nq = min(AQ, M - mq0);
     const int nk = pos0 + mq0 + nq;          // keys visible to the last query of the block
     const int nk_pad = (nk + 63) & ~63;      // <= s_stride - 8
@@ -668,97 +689,157 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, c
         for (int f = 0; f < 8; f++) qf[f] = *reinterpret_cast<const h16x8*>(qrow + f * 16);
     }
     {
-        // each wave takes key blocks wave, wave + 4, ...; the next block's rows are requested before this one is multiplied
-        auto load_k = [&](h16x8 (&kf)[8], int kb) {
-            const uint16_t* krow = kh + (size_t)min(kb * 32 + l32, nk - 1) * kv_dim + lh * 8;
+        // Each wave takes key blocks wave, wave + 4, ...; the rows of four of them are requested at once (512 keys are
+        // one round trip to memory per wave).  The rows are loaded as they lie in memory, 16 lanes x 16 bytes per
+        // 256-byte row, and turned into MFMA fragments through a tile of LDS private to the wave (the value tiles'
+        // space, idle until phase 3): loaded straight as fragments, an instruction touches 32 rows with 32 bytes each,
+        // and the address path of the compute unit takes twice as long over it (measured: 7 of the kernel's 20 us).
+        // Every load is unconditional, rows past the end clamped to the last one: a load inside a branch is waited
+        // for before the next one is issued.
+        constexpr int KU = 4;
+        uint16_t* kt = Vt + wave * (32 * KT_STRIDE);
+        const int crow = lane >> 4, cpiece = lane & 15;
+        for (int kb0 = wave; kb0 * 32 < nk_pad; kb0 += 4 * KU) {
+            u32x4 kr[KU][8];
 #pragma unroll
-            for (int f = 0; f < 8; f++) kf[f] = *reinterpret_cast<const h16x8*>(krow + f * 16);
-        };
-        h16x8 kf[8], kn[8];
-        if (wave * 32 < nk_pad) load_k(kf, wave);
-        for (int kb = wave; kb * 32 < nk_pad; kb += 4) {
-            const bool more = (kb + 4) * 32 < nk_pad;
-            if (more) load_k(kn, kb + 4);
-            f32x16 acc;
+            for (int u = 0; u < KU; u++) {
 #pragma unroll
-            for (int j = 0; j < 16; j++) acc[j] = 0.0f;
-#pragma unroll
-            for (int f = 0; f < 8; f++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[f], kf[f], acc, 0, 0, 0);
-#pragma unroll
-            for (int j = 0; j < 16; j++) {
-                const int row = (j >> 2) * 8 + lh * 4 + (j & 3);
-                S[row * s_stride + kb * 32 + l32] = float_to_half_bits(acc[j] * alpha);
+                for (int r = 0; r < 8; r++) {
+                    const int key = min((kb0 + 4 * u) * 32 + r * 4 + crow, nk - 1);
+                    kr[u][r] = *reinterpret_cast<const u32x4*>(kh + (size_t)key * kv_dim + cpiece * 8);
+                }
             }
-            if (more) {
+            // (the compiler would otherwise move some of these loads down to their use, one wait each)
 #pragma unroll
-                for (int f = 0; f < 8; f++) kf[f] = kn[f];
+            for (int u = 0; u < KU; u++)
+#pragma unroll
+                for (int r = 0; r < 8; r++) asm volatile("" : "+v"(kr[u][r]));
+#pragma unroll
+            for (int u = 0; u < KU; u++) {
+                const int kb = kb0 + 4 * u;
+                if (kb * 32 < nk_pad) {
+#pragma unroll
+                    for (int r = 0; r < 8; r++)
+                        *reinterpret_cast<u32x4*>(kt + (r * 4 + crow) * KT_STRIDE + cpiece * 8) = kr[u][r];
+                    __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order; this keeps the compiler from reordering them
+                    h16x8 kf[8];
+#pragma unroll
+                    for (int f = 0; f < 8; f++) kf[f] = *reinterpret_cast<const h16x8*>(kt + l32 * KT_STRIDE + f * 16 + lh * 8);
+                    __builtin_amdgcn_wave_barrier();
+                    f32x16 acc;
+#pragma unroll
+                    for (int j = 0; j < 16; j++) acc[j] = 0.0f;
+#pragma unroll
+                    for (int f = 0; f < 8; f++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(qf[f], kf[f], acc, 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < 16; j++) {
+                        const int row = (j >> 2) * 8 + lh * 4 + (j & 3);
+                        S[row * s_stride + kb * 32 + l32] = float_to_half_bits(acc[j] * alpha);
+                    }
+                }
             }
         }
     }
+    // O = P V below stages the value rows through LDS, 8 keys x 8 dimensions per thread transposed in registers: the
+    // waves 0-1 take the first 64 keys of a block of 128, the waves 2-3 the second.  The first two blocks are requested
+    // here, so that they arrive while the softmax runs.
+    const int kg = tid & 7, dc = (tid >> 3) & 15, vhalf = tid >> 7;
+    u32x4 va[8], vb[8];
+    auto load_v = [&](u32x4 (&vr)[8], int t0) {  // unconditional, rows past the end clamped
+#pragma unroll
+        for (int r = 0; r < 8; r++)
+            vr[r] = *reinterpret_cast<const u32x4*>(vh + (size_t)min(t0 + vhalf * 64 + kg * 8 + r, nk - 1) * kv_dim + dc * 8);
+    };
+    load_v(va, 0);
+    load_v(vb, 128);
     __syncthreads();
-    // 2. softmax per query row (wave w takes rows w, w+4, ...); rows past nq get all-zero probabilities
-    for (int qi = wave; qi < AQ; qi += 4) {
+    // 2. softmax per query row; rows past nq get all-zero probabilities
+    if (nk_pad <= 512) {
+        // Eight lanes per row, the eight rows of a wave side by side: a lane holds up to 64 scores of its row in
+        // registers (16-byte LDS accesses, one exponential per score), and the row's maximum and sum are reductions
+        // over 8 lanes.  Row by row with the wave across one row, each row is a chain of dependent reductions with
+        // nothing to overlap it (measured: 7 us for 32 rows of 32 scores).
+        const int r8 = lane >> 3, l8 = lane & 7;
+        const int qi = wave * 8 + r8;
         const int size = qi < nq ? pos0 + mq0 + qi + 1 : 0;
         uint16_t* srow = S + qi * s_stride;
+        const int iters = nk_pad >> 6;  // chunks of 8 scores per lane
+        float v[8][8];
         float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed
-        if (nk_pad <= 512) {
-            // up to 8 scores per lane stay in registers: one exponential per score instead of two
-            float v[8];
 #pragma unroll
-            for (int k = 0; k < 8; k++) {
-                const int t = lane + 64 * k;
-                v[k] = t < size ? half_bits_to_float(srow[t]) : -INFINITY;
-                m = fmaxf(m, v[k]);
-            }
-            m = wave_max(m);
-            float sum = 0.0f;
+        for (int i = 0; i < 8; i++) {
+            if (i < iters) {
+                const int t0 = (l8 + 8 * i) * 8;
+                const u32x4 raw = *reinterpret_cast<const u32x4*>(srow + t0);
 #pragma unroll
-            for (int k = 0; k < 8; k++) {
-                v[k] = lane + 64 * k < size ? expf(v[k] - m) : 0.0f;
-                sum += v[k];
+                for (int e = 0; e < 4; e++) {
+                    const h16x2 hh = as_h2(raw[e]);
+                    v[i][2 * e] = t0 + 2 * e < size ? (float)hh[0] : -INFINITY;
+                    v[i][2 * e + 1] = t0 + 2 * e + 1 < size ? (float)hh[1] : -INFINITY;
+                    m = fmaxf(m, fmaxf(v[i][2 * e], v[i][2 * e + 1]));
+                }
             }
-            sum = wave_sum(sum);
-#pragma unroll
-            for (int k = 0; k < 8; k++) {
-                const int t = lane + 64 * k;
-                if (t < nk_pad) srow[t] = float_to_half_bits(t < size ? v[k] / sum : 0.0f);
-            }
-            continue;
         }
-        for (int t = lane; t < size; t += 64) m = fmaxf(m, half_bits_to_float(srow[t]));
-        m = wave_max(m);
+        m = fmaxf(m, dpp_mov<0xB1>(m));
+        m = fmaxf(m, dpp_mov<0x4E>(m));
+        m = fmaxf(m, dpp_mov<0x141>(m));
         float sum = 0.0f;
-        for (int t = lane; t < size; t += 64) sum += expf(half_bits_to_float(srow[t]) - m);
-        sum = wave_sum(sum);
-        for (int t = lane; t < nk_pad; t += 64) {
-            float pv = 0.0f;
-            if (t < size) pv = expf(half_bits_to_float(srow[t]) - m) / sum;
-            srow[t] = float_to_half_bits(pv);
-        }
-    }
-    // 3. O = P V.  Loader role (threads 0..127): 8 keys x 8 dims, transposed in registers.
-    const int kg = tid & 7, dc = (tid >> 3) & 15;
-    const bool loader = tid < 128;
-    // value rows travel two blocks of 64 keys ahead of the multiply, in two register sets
-    u32x4 va[8], vb[8];
-    auto load_v = [&](u32x4 (&vr)[8], int t0) {
-        if (loader) {
 #pragma unroll
-            for (int r = 0; r < 8; r++)
-                vr[r] = *reinterpret_cast<const u32x4*>(vh + (size_t)min(t0 + kg * 8 + r, nk - 1) * kv_dim + dc * 8);
-        }
-    };
-    auto store_v = [&](const u32x4 (&vr)[8], int buf) {
-        if (loader) {
-            uint16_t* vt = Vt + buf * (HS * VT_STRIDE);
+        for (int i = 0; i < 8; i++) {
+            if (i < iters) {
 #pragma unroll
-            for (int d = 0; d < 8; d++) {
-                const uint32_t sel = (d & 1) ? 0x07060302u : 0x05040100u;
+                for (int e = 0; e < 8; e++) {
+                    v[i][e] = expf(v[i][e] - m);  // exp(-inf) = 0 for the masked scores
+                    sum += v[i][e];
+                }
+            }
+        }
+        sum = group_sum<8>(sum);
+        if (size == 0) sum = 1.0f;  // a row past nq: all exponentials are zero, and so are the quotients
+        const float rcp = 1.0f / sum;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (i < iters) {
+                const int t0 = (l8 + 8 * i) * 8;
                 u32x4 o;
 #pragma unroll
-                for (int r2 = 0; r2 < 4; r2++) o[r2] = __builtin_amdgcn_perm(vr[2 * r2 + 1][d >> 1], vr[2 * r2][d >> 1], sel);
-                *reinterpret_cast<u32x4*>(&vt[(dc * 8 + d) * VT_STRIDE + kg * 8]) = o;
+                for (int e = 0; e < 4; e++) {
+                    h16x2 hh;
+                    hh[0] = (h16_t)quotient(v[i][2 * e], sum, rcp);  // masked scores: 0 / sum
+                    hh[1] = (h16_t)quotient(v[i][2 * e + 1], sum, rcp);
+                    o[e] = as_u32(hh);
+                }
+                *reinterpret_cast<u32x4*>(srow + t0) = o;
             }
+        }
+    } else {
+        for (int qi = wave; qi < AQ; qi += 4) {  // wave w takes rows w, w+4, ...
+            const int size = qi < nq ? pos0 + mq0 + qi + 1 : 0;
+            uint16_t* srow = S + qi * s_stride;
+            float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed
+            for (int t = lane; t < size; t += 64) m = fmaxf(m, half_bits_to_float(srow[t]));
+            m = wave_max(m);
+            float sum = 0.0f;
+            for (int t = lane; t < size; t += 64) sum += expf(half_bits_to_float(srow[t]) - m);
+            sum = wave_sum(sum);
+            for (int t = lane; t < nk_pad; t += 64) {
+                float pv = 0.0f;
+                if (t < size) pv = expf(half_bits_to_float(srow[t]) - m) / sum;
+                srow[t] = float_to_half_bits(pv);
+            }
+        }
+    }
+    // 3. O = P V, 128 keys per round: every thread transposes its 8 x 8 piece into the LDS tile of its half, then
+    // every wave multiplies both tiles.  Value rows travel two rounds ahead of the multiply, in two register sets.
+    auto store_v = [&](const u32x4 (&vr)[8]) {
+        uint16_t* vt = Vt + vhalf * (HS * VT_STRIDE);
+#pragma unroll
+        for (int d = 0; d < 8; d++) {
+            const uint32_t sel = (d & 1) ? 0x07060302u : 0x05040100u;
+            u32x4 o;
+#pragma unroll
+            for (int r2 = 0; r2 < 4; r2++) o[r2] = __builtin_amdgcn_perm(vr[2 * r2 + 1][d >> 1], vr[2 * r2][d >> 1], sel);
+            *reinterpret_cast<u32x4*>(&vt[(dc * 8 + d) * VT_STRIDE + kg * 8]) = o;
         }
     };
     f32x16 oacc;
@@ -773,21 +854,19 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(uint16_t* out, c
             oacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(pf, vf, oacc, 0, 0, 0);
         }
     };
-    load_v(va, 0);
-    if (64 < nk_pad) load_v(vb, 64);
-    store_v(va, 0);
-    if (128 < nk_pad) load_v(va, 128);
-    __syncthreads();  // also orders the probabilities written above
-    // blocks alternate between the register sets: block k (keys 64k ..) is in set k & 1 and LDS buffer k & 1
-    for (int t0 = 0; t0 < nk_pad; t0 += 128) {
+    for (int t0 = 0; t0 < nk_pad; t0 += 256) {
+        store_v(va);
+        load_v(va, t0 + 256);
+        __syncthreads();  // the first one also orders the probabilities written above
         multiply(t0, 0);
-        if (t0 + 64 < nk_pad) store_v(vb, 1);
-        if (t0 + 192 < nk_pad) load_v(vb, t0 + 192);
+        if (t0 + 64 < nk_pad) multiply(t0 + 64, 1);
+        __syncthreads();  // every wave is done with the tiles before they are overwritten
+        if (t0 + 128 >= nk_pad) break;
+        store_v(vb);
+        load_v(vb, t0 + 384);
         __syncthreads();
-        if (t0 + 64 >= nk_pad) break;
-        multiply(t0 + 64, 1);
-        if (t0 + 128 < nk_pad) store_v(va, 0);
-        if (t0 + 256 < nk_pad) load_v(va, t0 + 256);
+        multiply(t0 + 128, 0);
+        if (t0 + 192 < nk_pad) multiply(t0 + 192, 1);
         __syncthreads();
     }
 #pragma unroll
@@ -1027,7 +1106,7 @@ int awq_launch_attn_prefill(awq_ctx* ctx, uint16_t* out, const uint16_t* q, cons
                 return AWQ_ERR_HIP;
             }
         }
-        hipLaunchKernelGGL(pf::attn_prefill_mfma_kernel, dim3(div_up(M, pf::AQ), nh), dim3(256), lds, ctx->stream, out, q, kc, vc,
+        hipLaunchKernelGGL(pf::attn_prefill_mfma_kernel, dim3(8 * ((nh + 7) / 8) * div_up(M, pf::AQ)), dim3(256), lds, ctx->stream, out, q, kc, vc,
                            nh, kv_mul, M, pos0, s_stride, out_perm);
         return awq_check_launch("attn_prefill_mfma");
     }
