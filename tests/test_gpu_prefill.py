@@ -47,7 +47,13 @@ CFG_GQA = dict(dim=512, hidden_dim=1280, n_layers=2, n_heads=8, n_kv_heads=2, vo
 CFG_GQA128 = dict(dim=1024, hidden_dim=1536, n_layers=2, n_heads=8, n_kv_heads=2, vocab_size=512, seq_len=128, rope_theta=10000.0)
 
 
-@pytest.mark.parametrize("cfg,n_prompt", [(CFG, 130), (CFG, 16), (CFG, 1), (CFG, 97), (CFG_GQA, 70), (CFG_GQA128, 75)])
+# 128-wide heads and a prompt longer than one 512-token chunk: the second chunk attends to more than 512 keys (several
+# rounds of key blocks per wave, the two-pass softmax, more than two rounds of value tiles)
+CFG_LONG128 = dict(dim=256, hidden_dim=512, n_layers=2, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=1024, rope_theta=10000.0)
+
+
+@pytest.mark.parametrize("cfg,n_prompt", [(CFG, 130), (CFG, 16), (CFG, 1), (CFG, 97), (CFG_GQA, 70), (CFG_GQA128, 75),
+                                          (CFG_LONG128, 700), (CFG_LONG128, 1000)])
 def test_prefill_matches_token_by_token_oracle(ctx, cfg, n_prompt):
     img = synth.make_model_image(cfg, seed=31)
     t = A.Transformer(ctx, image=img)
