@@ -813,20 +813,59 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(uint16_t* out
             }
         }
     } else {
-        for (int qi = wave; qi < AQ; qi += 4) {  // wave w takes rows w, w+4, ...
-            const int size = qi < nq ? pos0 + mq0 + qi + 1 : 0;
-            uint16_t* srow = S + qi * s_stride;
-            float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed
-            for (int t = lane; t < size; t += 64) m = fmaxf(m, half_bits_to_float(srow[t]));
-            m = wave_max(m);
-            float sum = 0.0f;
-            for (int t = lane; t < size; t += 64) sum += expf(half_bits_to_float(srow[t]) - m);
-            sum = wave_sum(sum);
-            for (int t = lane; t < nk_pad; t += 64) {
-                float pv = 0.0f;
-                if (t < size) pv = expf(half_bits_to_float(srow[t]) - m) / sum;
-                srow[t] = float_to_half_bits(pv);
+        // More than 512 keys: the same layout, with the scores read from LDS again in each of the three passes
+        // (maximum, sum of exponentials, probabilities) instead of kept in registers.
+        const int r8 = lane >> 3, l8 = lane & 7;
+        const int qi = wave * 8 + r8;
+        const int size = qi < nq ? pos0 + mq0 + qi + 1 : 0;
+        uint16_t* srow = S + qi * s_stride;
+        const int iters = nk_pad >> 6;
+        auto scores8 = [&](int i, float (&x)[8]) {  // the lane's i-th chunk of 8 scores, masked ones as -inf
+            const int t0 = (l8 + 8 * i) * 8;
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(srow + t0);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const h16x2 hh = as_h2(raw[e]);
+                x[2 * e] = t0 + 2 * e < size ? (float)hh[0] : -INFINITY;
+                x[2 * e + 1] = t0 + 2 * e + 1 < size ? (float)hh[1] : -INFINITY;
             }
+        };
+        float m = (size < 1024) ? 0.0f : -INFINITY;  // the reference's idle-lane seed
+#pragma unroll 4
+        for (int i = 0; i < iters; i++) {
+            float x[8];
+            scores8(i, x);
+#pragma unroll
+            for (int e = 0; e < 8; e++) m = fmaxf(m, x[e]);
+        }
+        m = fmaxf(m, dpp_mov<0xB1>(m));
+        m = fmaxf(m, dpp_mov<0x4E>(m));
+        m = fmaxf(m, dpp_mov<0x141>(m));
+        if (size == 0) m = 0.0f;  // a row past nq (with the -inf seed of long contexts): keep exp(-inf - m) defined
+        float sum = 0.0f;
+#pragma unroll 2
+        for (int i = 0; i < iters; i++) {
+            float x[8];
+            scores8(i, x);
+#pragma unroll
+            for (int e = 0; e < 8; e++) sum += expf(x[e] - m);
+        }
+        sum = group_sum<8>(sum);
+        if (size == 0) sum = 1.0f;
+        const float rcp = 1.0f / sum;
+#pragma unroll 2
+        for (int i = 0; i < iters; i++) {
+            float x[8];
+            scores8(i, x);
+            u32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                h16x2 hh;
+                hh[0] = (h16_t)quotient(expf(x[2 * e] - m), sum, rcp);
+                hh[1] = (h16_t)quotient(expf(x[2 * e + 1] - m), sum, rcp);
+                o[e] = as_u32(hh);
+            }
+            *reinterpret_cast<u32x4*>(srow + (l8 + 8 * i) * 8) = o;
         }
     }
     // 3. O = P V, 128 keys per round: every thread transposes its 8 x 8 piece into the LDS tile of its half, then
