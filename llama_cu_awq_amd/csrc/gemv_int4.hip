@@ -79,11 +79,22 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     constexpr int NS = (KIND == KIND_FFN) ? 2 * R : R;
     const Int4Mat m0 = (KIND == KIND_QKV) ? (which == 0 ? p.m[0] : (which == 1 ? p.m[1] : p.m[2])) : p.m[0];
     const Int4Mat m1 = p.m[1];  // FFN: up
-    uint16_t* out = (KIND == KIND_QKV) ? (which == 0 ? p.out[0] : (which == 1 ? p.out[1] : p.out[2])) : p.out[0];
-    {
-        const int loff = (KIND == KIND_QKV) ? (which == 0 ? p.loff[0] : (which == 1 ? p.loff[1] : p.loff[2])) : p.loff[0];
-        if (loff != -1) out += (size_t)loff + (size_t)(*p.pos) * p.N;
+    uint16_t* out_base = (KIND == KIND_QKV) ? (which == 0 ? p.out[0] : (which == 1 ? p.out[1] : p.out[2])) : p.out[0];
+    // The position (row of the KV cache, rotation angle) is only needed in the epilogue.  Read as a scalar it is waited
+    // for right here, a round trip before anything else is requested; read as the kernel's first vector load (through
+    // an address the compiler cannot prove uniform) it returns ahead of everything else and nothing waits for it.
+    int loff = (KIND == KIND_QKV) ? (which == 0 ? p.loff[0] : (which == 1 ? p.loff[1] : p.loff[2])) : p.loff[0];
+    if (RES && p.accum && loff != -1) {
+        // adding to a row that depends on the position: the old values are requested along with the weights
+        out_base += (size_t)loff + (size_t)(*p.pos) * p.N;
+        loff = -1;
     }
+    // (unconditional: a load inside a branch is waited for before the next one is issued; without a position the word
+    // read is the head of the packed weights, the one pointer every form of the kernel has, and goes unused)
+    int zero = 0;
+    asm volatile("" : "+v"(zero));
+    const int* pos_word = p.pos ? p.pos : reinterpret_cast<const int*>(m0.w);
+    const int pos_now = pos_word[zero];
 
     // This workgroup's row groups (W waves x R rows each).  A wave walks its rows as a sequence of stages (group-major,
     // then pass); D stages are in flight at any time.  The sequence is padded to a multiple of D with repeats of the
@@ -105,7 +116,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
         for (int r = 0; r < R; r++) {
             const int li = min((g * W + wave) * R + r, p.N - 1);  // indices past N are recomputed, never stored
             const int row = rope_here ? map_row<true>(li, p.head_size) : li;
-            resrow[r] = out + row;
+            resrow[r] = out_base + row;  // (the residual form never writes KV-cache rows: no position offset)
             if (KIND == KIND_FFN) {
                 wrow[2 * r] = m0.w + (size_t)row * pwh;
                 zrow[2 * r] = m0.z + (size_t)row * p.pzh;
@@ -157,10 +168,12 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
         for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]) * kChunkDotUnscale;  // chunk_dot works in units of 2^-24
         const int li0 = (cg * W + wave) * R;
         if (lane == 0 && li0 < p.N) {
+            uint16_t* out = out_base;
+            if (loff != -1) out += (size_t)loff + (size_t)pos_now * p.N;
             if (rope_here) {
                 // q/k are rounded to fp16 and then rotated, as the separate RoPE kernel does (gpu_kernels.h:351-361)
                 const int half = p.head_size >> 1;
-                const float2* cs_tab = p.rope + (size_t)(*p.pos) * half;
+                const float2* cs_tab = p.rope + (size_t)pos_now * half;
 #pragma unroll
                 for (int r = 0; r + 1 < R; r += 2) {
                     const int li = li0 + r;
