@@ -61,7 +61,12 @@ __device__ __forceinline__ int map_row(int li, int head_size) {
     return (pi / half) * head_size + (pi % half) + (li & 1) * half;
 }
 
-template <int W, int R, int D, int KIND, bool NORM, bool ROPE, bool PARTS = false>
+// HALF: a row takes 32 lanes instead of 64, and the two halves of a wave work on two rows (QKV with RoPE: the two rows of
+// a rotation pair; FFN: two gate/up pairs) side by side, so a pass covers 32 chunks of each.  A row whose chunk count
+// leaves at most half a 64-lane pass over (K = 5120: 2.5 passes, 6656: 3.25, 11008: 5.375) then takes ceil(C / 32)
+// passes per two rows instead of 2 * ceil(C / 64): the kernels' time follows the number of passes, not the bytes
+// (K = 11008 and K = 12288 took the same 6.9 us; 10240: 6.4).  R then counts the row pairs of a wave.
+template <int W, int R, int D, int KIND, bool NORM, bool ROPE, bool PARTS = false, bool HALF = false>
 __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     static_assert(!PARTS || (!NORM && KIND == KIND_SINGLE), "partial-sum input only for the plain single-matrix form");
     extern __shared__ u32x4 xs[];
@@ -70,7 +75,11 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: row addresses stay scalar
     const int C = p.C;
     const int pwh = C * 4;
-    const int P = (C + 63) >> 6;  // 64-lane passes per row
+    constexpr int LPR = HALF ? 32 : 64;   // lanes per row
+    constexpr int RW = HALF ? 2 * R : R;  // rows (FFN: gate/up pairs) of a wave per row group
+    const int hf = HALF ? lane >> 5 : 0;   // which of the wave's two rows this lane works on
+    const int ll = HALF ? lane & 31 : lane;
+    const int P = (C + LPR - 1) / LPR;  // passes per row (HALF: per two rows)
     float* ca = reinterpret_cast<float*>(xs + 4 * C);
     const int which = (KIND == KIND_QKV) ? blockIdx.y : 0;
     const bool rope_here = ROPE && which != 2;
@@ -101,7 +110,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     // last stage, which are loaded (same addresses again) but not accumulated, so that the number of loads between a
     // stage's request and its use is a compile-time constant.
     // The workgroup takes row groups blockIdx.x, blockIdx.x + gridDim.x, ... (x is staged once for all of them).
-    const int groups_total = (p.N + W * R - 1) / (W * R);
+    const int groups_total = (p.N + W * RW - 1) / (W * RW);
     const int g_begin = blockIdx.x, g_stride = gridDim.x;
     const int total = ((groups_total - 1 - g_begin) / g_stride + 1) * P;
 
@@ -110,12 +119,23 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     const uint32_t* zrow[NS];
     const uint16_t* srow[NS];
     const uint16_t* resrow[R];
+    // HALF: the row pointers are those of the lower half's row; the upper half adds the distance to its own row
+    // (0 when both indices are clamped to the last row), as byte offsets on top of the lane's offset in the row
+    uint32_t hoff_w[R], hoff_z[R], hoff_s[R], hoff_r[R];
     int lg = g_begin, lp = 0, ls = 0;
     auto set_rows = [&](int g) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const int li = min((g * W + wave) * R + r, p.N - 1);  // indices past N are recomputed, never stored
+            const int li = min((g * W + wave) * RW + (HALF ? 2 * r : r), p.N - 1);  // indices past N are recomputed, never stored
             const int row = rope_here ? map_row<true>(li, p.head_size) : li;
+            if (HALF) {
+                const int li_up = min((g * W + wave) * RW + 2 * r + 1, p.N - 1);
+                const int drow = (rope_here ? map_row<true>(li_up, p.head_size) : li_up) - row;
+                hoff_w[r] = hf ? (uint32_t)(drow * pwh * 4) : 0u;
+                hoff_z[r] = hf ? (uint32_t)(drow * p.pzh * 4) : 0u;
+                hoff_s[r] = hf ? (uint32_t)(drow * p.sh * 2) : 0u;
+                hoff_r[r] = hf ? (uint32_t)(drow * 2) : 0u;
+            }
             resrow[r] = out_base + row;  // (the residual form never writes KV-cache rows: no position offset)
             if (KIND == KIND_FFN) {
                 wrow[2 * r] = m0.w + (size_t)row * pwh;
@@ -132,19 +152,22 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
         }
     };
     auto issue = [&](Stage<NS>& st) {
-        const int c = min(lp * 64 + lane, C - 1);  // lanes past the row end repeat its last chunk; consume() drops them
+        const int c = min(lp * LPR + ll, C - 1);  // lanes past the row end repeat its last chunk; consume() drops them
         // byte offsets as unsigned 32-bit values on top of wave-uniform row pointers: the loads take the scalar-base
         // form and need no 64-bit address arithmetic per lane
         const uint32_t off_w = (uint32_t)c << 4, off_z = (uint32_t)(c >> 5) << 2, off_s = (uint32_t)(c >> 2) << 1;
 #pragma unroll
         for (int i = 0; i < NS; i++) {
-            st.w[i] = load_nt(reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(wrow[i]) + off_w));
-            st.zw[i] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(zrow[i]) + off_z);
-            st.s[i] = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(srow[i]) + off_s);
+            const int r = (KIND == KIND_FFN) ? i >> 1 : i;  // gate and up of a pair are the same row of two matrices
+            const uint32_t ow = HALF ? off_w + hoff_w[r] : off_w, oz = HALF ? off_z + hoff_z[r] : off_z, os = HALF ? off_s + hoff_s[r] : off_s;
+            st.w[i] = load_nt(reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(wrow[i]) + ow));
+            st.zw[i] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(zrow[i]) + oz);
+            st.s[i] = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(srow[i]) + os);
         }
         if (RES) {
 #pragma unroll
-            for (int r = 0; r < R; r++) st.res[r] = *resrow[r];
+            for (int r = 0; r < R; r++)
+                st.res[r] = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(resrow[r]) + (HALF ? hoff_r[r] : 0u));
         }
         ls++;
         if (ls < total) {
@@ -164,23 +187,29 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     // ---- consume cursor
     int cg = g_begin, cp = 0, cs = 0;
     auto finish_group = [&](const Stage<NS>& st) {
+        // chunk_dot works in units of 2^-24; with HALF every lane ends up with the sum of its own half of the wave
 #pragma unroll
-        for (int i = 0; i < NS; i++) sum[i] = wave_sum(sum[i]) * kChunkDotUnscale;  // chunk_dot works in units of 2^-24
-        const int li0 = (cg * W + wave) * R;
-        if (lane == 0 && li0 < p.N) {
-            uint16_t* out = out_base;
-            if (loff != -1) out += (size_t)loff + (size_t)pos_now * p.N;
-            if (rope_here) {
-                // q/k are rounded to fp16 and then rotated, as the separate RoPE kernel does (gpu_kernels.h:351-361)
+        for (int i = 0; i < NS; i++)
+            sum[i] = (HALF ? lane_xor_sum<16>(row16_sum(sum[i])) : wave_sum(sum[i])) * kChunkDotUnscale;
+        const int li0 = (cg * W + wave) * RW;
+        if (rope_here) {
+            // q/k are rounded to fp16 and then rotated, as the separate RoPE kernel does (gpu_kernels.h:351-361);
+            // the two rows of a pair are two streams of the wave, or (HALF) its two halves
+            float second[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) second[r] = HALF ? read_lane(sum[r], 32) : 0.0f;
+            if (lane == 0 && li0 < p.N) {
+                uint16_t* out = out_base;
+                if (loff != -1) out += (size_t)loff + (size_t)pos_now * p.N;
                 const int half = p.head_size >> 1;
                 const float2* cs_tab = p.rope + (size_t)pos_now * half;
 #pragma unroll
-                for (int r = 0; r + 1 < R; r += 2) {
-                    const int li = li0 + r;
+                for (int r = 0; r < (HALF ? R : R - 1); r += (HALF ? 1 : 2)) {
+                    const int li = li0 + (HALF ? 2 * r : r);
                     if (li < p.N) {
                         const int row = map_row<true>(li, p.head_size);
                         const float v0 = half_bits_to_float(float_to_half_bits(sum[r]));
-                        const float v1 = half_bits_to_float(float_to_half_bits(sum[r + 1]));
+                        const float v1 = half_bits_to_float(float_to_half_bits(HALF ? second[r] : sum[HALF ? r : r + 1]));
                         const float2 c = cs_tab[row % half];
                         float r0, r1;
                         rope_rotate(v0, v1, c.x, c.y, r0, r1);
@@ -188,23 +217,25 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
                         out[row + half] = float_to_half_bits(r1);
                     }
                 }
-            } else {
+            }
+        } else if (ll == 0) {
+            uint16_t* out = out_base;
+            if (loff != -1) out += (size_t)loff + (size_t)pos_now * p.N;
 #pragma unroll
-                for (int r = 0; r < R; r++) {
-                    const int row = li0 + r;
-                    if (row < p.N) {
-                        float v;
-                        if (KIND == KIND_FFN) {
-                            // gate = stream 2r, up = stream 2r+1 (gpu_kernels.h:276-281)
-                            float g = sum[2 * r];
-                            g *= 1.0f / (1.0f + expf(-g));
-                            v = g * sum[2 * r + 1];
-                        } else {
-                            v = sum[r];
-                            if (RES && p.accum) v += half_bits_to_float(st.res[r]) * p.inv_gpu_count;
-                        }
-                        out[row] = float_to_half_bits(v);
+            for (int r = 0; r < R; r++) {
+                const int row = li0 + (HALF ? 2 * r + hf : r);
+                if (row < p.N) {
+                    float v;
+                    if (KIND == KIND_FFN) {
+                        // gate = stream 2r, up = stream 2r+1 (gpu_kernels.h:276-281)
+                        float g = sum[2 * r];
+                        g *= 1.0f / (1.0f + expf(-g));
+                        v = g * sum[2 * r + 1];
+                    } else {
+                        v = sum[r];
+                        if (RES && p.accum) v += half_bits_to_float(st.res[r]) * p.inv_gpu_count;
                     }
+                    out[row] = float_to_half_bits(v);
                 }
             }
         }
@@ -213,7 +244,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     };
     auto consume = [&](const Stage<NS>& st) {
         if (cs < total) {
-            const int c = cp * 64 + lane;
+            const int c = cp * LPR + ll;
             const int cc = min(c, C - 1);
             u32x4 xq[4];
 #pragma unroll
@@ -330,9 +361,9 @@ struct GemvPlan {
     int depth;   // stages in flight per wave (2, 3, 4)
 };
 
-template <int W, int R, int D, int KIND, bool ROPE>
+template <int W, int R, int D, int KIND, bool ROPE, bool HALF = false>
 int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
-    const int groups_total = div_up(p.N, W * R);
+    const int groups_total = div_up(p.N, W * R * (HALF ? 2 : 1));
     int gx = groups_total;
     // The norm-fused gate/up kernel stages (and normalises) x in every workgroup, and that work is what bounds it:
     // three 4-wave workgroups per compute unit walk the row groups between them (measured best at the 7B shape; the
@@ -352,7 +383,7 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
     if constexpr (KIND == KIND_SINGLE && !ROPE && R == 1 && (W == 8 || W == 16)) {
         if (p.xpart) {
-            awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, false, true>, grid, dim3(W * 64), lds, p);
+            awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, false, true, HALF>, grid, dim3(W * 64), lds, p);
             return awq_check_launch(what);
         }
     }
@@ -361,10 +392,17 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
         return AWQ_ERR_ARG;
     }
     if (p.norm_w)
-        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, true, ROPE>, grid, dim3(W * 64), lds, p);
+        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, true, ROPE, false, HALF>, grid, dim3(W * 64), lds, p);
     else
-        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, ROPE>, grid, dim3(W * 64), lds, p);
+        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, ROPE, false, HALF>, grid, dim3(W * 64), lds, p);
     return awq_check_launch(what);
+}
+
+// The half-wave forms: one row pair per wave (two gate/up pairs in the FFN form), `depth` passes of the pair in flight.
+template <int W, int KIND, bool ROPE>
+int dispatch_half(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, int depth) {
+    if (depth == 2) return launch<W, 1, 2, KIND, ROPE, true>(ctx, p, grid_y, what);
+    return launch<W, 1, 3, KIND, ROPE, true>(ctx, p, grid_y, what);
 }
 
 template <int W, int R, int KIND, bool ROPE>
@@ -399,6 +437,16 @@ template <int KIND, bool ROPE>
 int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan plan) {
     if (p.norm_w && KIND == KIND_FFN && p.K <= 8192) plan.waves = 4;  // see launch()
     if (ROPE && plan.rows < 2) plan.rows = 2;  // a rotation pair lives in one wave
+    // Rows that leave at most half of a 64-lane pass over go two to a wave, 32 lanes each (see the kernel).  Measured
+    // at the 13B and 33B shapes (K = 5120, 6656): gate/up -6 %, O projection -7 %, QKV -2 % with two passes in flight
+    // and even with three, tokens/s +3 %.  Rows above 8192 (K = 11008: 16 waves, or 8, at any depth) lose: two rows per
+    // wave halve the workgroups of a matrix that has few rows to begin with.
+    const int tail = p.C & 63;
+    if (tail != 0 && tail <= 32 && plan.rows <= 2 && p.K <= 8192) {
+        const int depth = KIND == KIND_QKV ? 2 : 3;
+        if (plan.waves == 4) return dispatch_half<4, KIND, ROPE>(ctx, p, grid_y, what, depth);
+        return dispatch_half<8, KIND, ROPE>(ctx, p, grid_y, what, depth);
+    }
 #define AWQ_CASE(W_, R_) \
     if (plan.waves == W_ && plan.rows == R_) return dispatch_depth<W_, R_, KIND, ROPE>(ctx, p, grid_y, what, plan);
     AWQ_CASE(4, 2) AWQ_CASE(4, 4) AWQ_CASE(8, 2) AWQ_CASE(8, 4) AWQ_CASE(16, 2)
