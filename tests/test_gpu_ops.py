@@ -57,8 +57,8 @@ def test_matvec_int4_plain(ctx, K, N):
     assert rel_l2(got, f16(want)) <= 3e-4
 
 
-def test_matvec_int4_accum_and_kv_offset(ctx):
-    K, N = 4096, 4096
+@pytest.mark.parametrize("K,N", [(4096, 4096), (5120, 5120), (6656, 264), (416, 40)])  # 64-lane rows; two rows per wave
+def test_matvec_int4_accum_and_kv_offset(ctx, K, N):
     w, z, s, x = _case(K, N, 1)
     qw = A.QWeight.upload(ctx, w, z, s)
     dx = ctx.upload(x)
