@@ -451,17 +451,16 @@ __global__ __launch_bounds__(256) void gemv_f16_kernel(uint16_t* out, const uint
 #pragma unroll
     for (int r = 0; r < R; r++) sum[r] = 0.0f;
 
+    // Two batches of R x 16 bytes per lane in flight.  Every load is unconditional, pieces past the row end clamped to
+    // its last one (their products are skipped): a load inside a branch is waited for, together with everything
+    // requested before it, before the next one is issued.
     u32x4 a[R], b[R];
-    if (lane < n8) {
 #pragma unroll
-        for (int r = 0; r < R; r++) a[r] = load_nt(wrow[r] + lane);
-    }
+    for (int r = 0; r < R; r++) a[r] = load_nt(wrow[r] + min(lane, n8 - 1));
     for (int c = lane; c < n8 + lane; c += 128) {
         const int c1 = c + 64, c2 = c + 128;
-        if (c1 < n8) {
 #pragma unroll
-            for (int r = 0; r < R; r++) b[r] = load_nt(wrow[r] + c1);
-        }
+        for (int r = 0; r < R; r++) b[r] = load_nt(wrow[r] + min(c1, n8 - 1));
         if (c < n8) {
             const u32x4 xv = xs[c];
 #pragma unroll
@@ -469,10 +468,8 @@ __global__ __launch_bounds__(256) void gemv_f16_kernel(uint16_t* out, const uint
 #pragma unroll
                 for (int i = 0; i < 4; i++) sum[r] = dot2(a[r][i], xv[i], sum[r]);
         }
-        if (c2 < n8) {
 #pragma unroll
-            for (int r = 0; r < R; r++) a[r] = load_nt(wrow[r] + c2);
-        }
+        for (int r = 0; r < R; r++) a[r] = load_nt(wrow[r] + min(c2, n8 - 1));
         if (c1 < n8) {
             const u32x4 xv = xs[c1];
 #pragma unroll
@@ -512,10 +509,7 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* x, int siz
     for (int e0 = 0; e0 < n8; e0 += 4 * 1024) {
         u32x4 v[4];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int e = e0 + k * 1024 + tid;
-            if (e < n8) v[k] = x8[e];
-        }
+        for (int k = 0; k < 4; k++) v[k] = x8[min(e0 + k * 1024 + tid, n8 - 1)];  // unconditional: all four in flight together
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const int e = e0 + k * 1024 + tid;
