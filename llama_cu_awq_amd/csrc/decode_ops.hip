@@ -396,6 +396,18 @@ __global__ __launch_bounds__(256) void gemv_f16_kernel(uint16_t* out, const uint
     const int tid = threadIdx.x;
     const int n8 = n >> 3;
     const u32x4* xg = reinterpret_cast<const u32x4*>(x);
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int row0 = (blockIdx.x * 4 + wave) * R;
+    // The first batch of the wave's rows is requested before x is staged: the rows do not depend on x, and their way
+    // from memory overlaps the staging (rows past d are clamped to the last one and never stored).
+    const u32x4* wrow[R];
+    u32x4 a[R], b[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        wrow[r] = reinterpret_cast<const u32x4*>(w + (size_t)min(row0 + r, d - 1) * n);
+        a[r] = load_nt(wrow[r] + min(lane, n8 - 1));
+    }
     float ss = 0.0f;
     if (NORM) {
         float part = 0.0f;
@@ -440,13 +452,7 @@ __global__ __launch_bounds__(256) void gemv_f16_kernel(uint16_t* out, const uint
         for (int e = tid; e < n8; e += 256) reinterpret_cast<u32x4*>(norm_out)[e] = xs[e];
     }
 
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int row0 = (blockIdx.x * 4 + wave) * R;
     if (row0 >= d) return;
-    const u32x4* wrow[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) wrow[r] = reinterpret_cast<const u32x4*>(w + (size_t)min(row0 + r, d - 1) * n);
     float sum[R];
 #pragma unroll
     for (int r = 0; r < R; r++) sum[r] = 0.0f;
@@ -454,9 +460,6 @@ __global__ __launch_bounds__(256) void gemv_f16_kernel(uint16_t* out, const uint
     // Two batches of R x 16 bytes per lane in flight.  Every load is unconditional, pieces past the row end clamped to
     // its last one (their products are skipped): a load inside a branch is waited for, together with everything
     // requested before it, before the next one is issued.
-    u32x4 a[R], b[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) a[r] = load_nt(wrow[r] + min(lane, n8 - 1));
     for (int c = lane; c < n8 + lane; c += 128) {
         const int c1 = c + 64, c2 = c + 128;
 #pragma unroll
