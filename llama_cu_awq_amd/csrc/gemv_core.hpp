@@ -62,15 +62,20 @@ struct Stage {
 // staged (stage_x) while those are still on their way: XP pieces of 8 halves per thread travel in registers, the rest
 // of a longer vector is fetched late by stage_x itself.
 constexpr int XP = 2;
+// 4-wave workgroups carry four pieces per thread, so that vectors up to 8192 elements travel in registers whole (the late
+// fetch sits behind the staging barriers, one exposed round trip per 2048 elements: K = 5120 and 6656 at four waves),
+// 16-wave workgroups three (K = 17920).
+constexpr int pieces_for(int waves) { return waves <= 4 ? 4 : (waves >= 16 ? 3 : XP); }
 
-template <bool NORM>
+template <bool NORM, int NP = XP>
 struct XPieces {
-    u32x4 v[XP];
-    u32x4 w[NORM ? XP : 1];
+    u32x4 v[NP];
+    u32x4 w[NORM ? NP : 1];
 };
 
 template <int W, bool NORM>
-__device__ __forceinline__ void load_x(XPieces<NORM>& xr, const XArgs& p) {
+__device__ __forceinline__ void load_x(XPieces<NORM, pieces_for(W)>& xr, const XArgs& p) {
+    constexpr int XP = pieces_for(W);
     constexpr int T = W * 64;
     const int n8 = p.K >> 3;  // 8-half pieces of real data
     const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
@@ -199,7 +204,8 @@ __device__ __forceinline__ float piece_sumsq(u32x4 v, float part) {
 
 // red: W + 1 floats of LDS.
 template <int W, bool NORM>
-__device__ __forceinline__ void stage_x(u32x4* xs, float* ca, const XArgs& p, float* red, const XPieces<NORM>& xr) {
+__device__ __forceinline__ void stage_x(u32x4* xs, float* ca, const XArgs& p, float* red, const XPieces<NORM, pieces_for(W)>& xr) {
+    constexpr int XP = pieces_for(W);
     constexpr int T = W * 64;
     const int tid = threadIdx.x;
     const int n8 = p.K >> 3;

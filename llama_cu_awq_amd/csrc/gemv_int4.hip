@@ -271,7 +271,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     // The first D stages of packed weights are requested before x is staged, so that their HBM latency overlaps the
     // staging (and the RMSNorm reduction).
     const XArgs xa{p.x, p.norm_w, p.norm_out, p.K, p.C, p.xpart, p.xparts};
-    XPieces<NORM> xr;
+    XPieces<NORM, pieces_for(W)> xr;
     PartPieces pr;
     if constexpr (PARTS)
         load_parts<W>(pr, xa);
@@ -381,7 +381,7 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     }
     const dim3 grid(gx, grid_y);
     const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
-    if constexpr (KIND == KIND_SINGLE && !ROPE && R == 1 && (W == 8 || W == 16)) {
+    if constexpr (KIND == KIND_SINGLE && !ROPE && R == 1 && W == 8) {  // (partial-sum input comes with K <= 8192: 8 waves)
         if (p.xpart) {
             awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, false, true, HALF>, grid, dim3(W * 64), lds, p);
             return awq_check_launch(what);
