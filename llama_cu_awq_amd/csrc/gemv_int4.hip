@@ -361,6 +361,18 @@ struct GemvPlan {
     int depth;   // stages in flight per wave (2, 3, 4)
 };
 
+int compute_units() {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
 template <int W, int R, int D, int KIND, bool ROPE, bool HALF = false>
 int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     const int groups_total = div_up(p.N, W * R * (HALF ? 2 : 1));
@@ -369,14 +381,7 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     // three 4-wave workgroups per compute unit walk the row groups between them (measured best at the 7B shape; the
     // plain kernels are faster with one group per workgroup).
     if (p.norm_w && KIND == KIND_FFN) {
-        static int cus = 0;
-        if (!cus) {
-            int dev = 0, n = 0;
-            if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-                cus = n;
-            else
-                cus = 256;
-        }
+        const int cus = compute_units();
         if (gx > 3 * cus) gx = 3 * cus;
     }
     const dim3 grid(gx, grid_y);
@@ -441,6 +446,14 @@ GemvPlan plan_for(int K, int rows) {
 template <int KIND, bool ROPE>
 int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan plan) {
     if (p.norm_w && KIND == KIND_FFN && p.K <= 8192) plan.waves = 4;  // see launch()
+    if (plan.waves == 16 && plan.rows == 1) {
+        // Long rows, one per wave: every workgroup is resident at once, so the kernel takes as long as the compute unit
+        // with the most workgroups.  16-wave workgroups suit 4096 rows on 256 compute units (one each); 5120 rows are
+        // 320 workgroups, two on a quarter of the compute units and one on the rest, and go better as 640 of 8 waves
+        // (13B down projection 11.2 -> 10.7 us); 6656 rows are as uneven either way and keep 16 (measured).
+        const double per_cu16 = (double)div_up(p.N, 16) / compute_units(), per_cu8 = (double)div_up(p.N, 8) / compute_units();
+        if (ceil(per_cu8) / per_cu8 < ceil(per_cu16) / per_cu16 - 0.05) plan.waves = 8;
+    }
     if (ROPE && plan.rows < 2) plan.rows = 2;  // a rotation pair lives in one wave
     // Rows that leave at most half of a 64-lane pass over go two to a wave, 32 lanes each (see the kernel).  Measured
     // at the 13B and 33B shapes (K = 5120, 6656): gate/up -6 %, O projection -7 %, QKV -2 % with two passes in flight
