@@ -61,12 +61,13 @@ __device__ __forceinline__ int map_row(int li, int head_size) {
     return (pi / half) * head_size + (pi % half) + (li & 1) * half;
 }
 
-// HALF: a row takes 32 lanes instead of 64, and the two halves of a wave work on two rows (QKV with RoPE: the two rows of
-// a rotation pair; FFN: two gate/up pairs) side by side, so a pass covers 32 chunks of each.  A row whose chunk count
-// leaves at most half a 64-lane pass over (K = 5120: 2.5 passes, 6656: 3.25, 11008: 5.375) then takes ceil(C / 32)
-// passes per two rows instead of 2 * ceil(C / 64): the kernels' time follows the number of passes, not the bytes
-// (K = 11008 and K = 12288 took the same 6.9 us; 10240: 6.4).  R then counts the row pairs of a wave.
-template <int W, int R, int D, int KIND, bool NORM, bool ROPE, bool PARTS = false, bool HALF = false>
+// SPLIT (1, 2 or 4): a row takes 64 / SPLIT lanes, and the SPLIT parts of a wave work on SPLIT rows side by side (QKV
+// with RoPE: rotation pairs; FFN: gate/up pairs), so a pass covers 64 / SPLIT chunks of each.  A row whose chunk count
+// leaves at most half (a quarter) of a 64-lane pass over (K = 5120: 2.5 passes, 11008: 5.375; K = 6656: 3.25) then
+// takes ceil(C * SPLIT / 64) passes per SPLIT rows instead of SPLIT * ceil(C / 64): the kernels' time follows the
+// number of passes, not the bytes (K = 11008 and K = 12288 took the same 6.9 us; 10240: 6.4).  R then counts the row
+// sets of a wave.
+template <int W, int R, int D, int KIND, bool NORM, bool ROPE, bool PARTS = false, int SPLIT = 1>
 __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     static_assert(!PARTS || (!NORM && KIND == KIND_SINGLE), "partial-sum input only for the plain single-matrix form");
     extern __shared__ u32x4 xs[];
@@ -75,11 +76,13 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: row addresses stay scalar
     const int C = p.C;
     const int pwh = C * 4;
-    constexpr int LPR = HALF ? 32 : 64;   // lanes per row
-    constexpr int RW = HALF ? 2 * R : R;  // rows (FFN: gate/up pairs) of a wave per row group
-    const int hf = HALF ? lane >> 5 : 0;   // which of the wave's two rows this lane works on
-    const int ll = HALF ? lane & 31 : lane;
-    const int P = (C + LPR - 1) / LPR;  // passes per row (HALF: per two rows)
+    static_assert(SPLIT == 1 || SPLIT == 2 || SPLIT == 4, "a row takes 64, 32 or 16 lanes");
+    constexpr bool HALF = SPLIT > 1;        // (the name from when two was the only split)
+    constexpr int LPR = 64 / SPLIT;        // lanes per row
+    constexpr int RW = SPLIT * R;          // rows (FFN: gate/up pairs) of a wave per row group
+    const int hf = HALF ? lane / LPR : 0;  // which of the wave's SPLIT rows this lane works on
+    const int ll = HALF ? lane % LPR : lane;
+    const int P = (C + LPR - 1) / LPR;  // passes per row (per SPLIT rows)
     float* ca = reinterpret_cast<float*>(xs + 4 * C);
     const int which = (KIND == KIND_QKV) ? blockIdx.y : 0;
     const bool rope_here = ROPE && which != 2;
@@ -119,22 +122,22 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     const uint32_t* zrow[NS];
     const uint16_t* srow[NS];
     const uint16_t* resrow[R];
-    // HALF: the row pointers are those of the lower half's row; the upper half adds the distance to its own row
-    // (0 when both indices are clamped to the last row), as byte offsets on top of the lane's offset in the row
+    // SPLIT > 1: the row pointers are those of the first part's row; the other parts add the distance to their own rows
+    // (0 when the indices are clamped to the last row), as byte offsets on top of the lane's offset in the row
     uint32_t hoff_w[R], hoff_z[R], hoff_s[R], hoff_r[R];
     int lg = g_begin, lp = 0, ls = 0;
     auto set_rows = [&](int g) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const int li = min((g * W + wave) * RW + (HALF ? 2 * r : r), p.N - 1);  // indices past N are recomputed, never stored
+            const int li = min((g * W + wave) * RW + SPLIT * r, p.N - 1);  // indices past N are recomputed, never stored
             const int row = rope_here ? map_row<true>(li, p.head_size) : li;
             if (HALF) {
-                const int li_up = min((g * W + wave) * RW + 2 * r + 1, p.N - 1);
-                const int drow = (rope_here ? map_row<true>(li_up, p.head_size) : li_up) - row;
-                hoff_w[r] = hf ? (uint32_t)(drow * pwh * 4) : 0u;
-                hoff_z[r] = hf ? (uint32_t)(drow * p.pzh * 4) : 0u;
-                hoff_s[r] = hf ? (uint32_t)(drow * p.sh * 2) : 0u;
-                hoff_r[r] = hf ? (uint32_t)(drow * 2) : 0u;
+                const int li_own = min((g * W + wave) * RW + SPLIT * r + hf, p.N - 1);
+                const int drow = (rope_here ? map_row<true>(li_own, p.head_size) : li_own) - row;
+                hoff_w[r] = (uint32_t)(drow * pwh * 4);
+                hoff_z[r] = (uint32_t)(drow * p.pzh * 4);
+                hoff_s[r] = (uint32_t)(drow * p.sh * 2);
+                hoff_r[r] = (uint32_t)(drow * 2);
             }
             resrow[r] = out_base + row;  // (the residual form never writes KV-cache rows: no position offset)
             if (KIND == KIND_FFN) {
@@ -187,25 +190,34 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     // ---- consume cursor
     int cg = g_begin, cp = 0, cs = 0;
     auto finish_group = [&](const Stage<NS>& st) {
-        // chunk_dot works in units of 2^-24; with HALF every lane ends up with the sum of its own half of the wave
+        // chunk_dot works in units of 2^-24; with SPLIT > 1 every lane ends up with the sum of its own part of the wave
 #pragma unroll
-        for (int i = 0; i < NS; i++)
-            sum[i] = (HALF ? lane_xor_sum<16>(row16_sum(sum[i])) : wave_sum(sum[i])) * kChunkDotUnscale;
+        for (int i = 0; i < NS; i++) {
+            float v = sum[i];
+            if (SPLIT == 1) v = wave_sum(v);
+            else if (SPLIT == 2) v = lane_xor_sum<16>(row16_sum(v));
+            else v = row16_sum(v);
+            sum[i] = v * kChunkDotUnscale;
+        }
         const int li0 = (cg * W + wave) * RW;
         if (rope_here) {
             // q/k are rounded to fp16 and then rotated, as the separate RoPE kernel does (gpu_kernels.h:351-361);
-            // the two rows of a pair are two streams of the wave, or (HALF) its two halves
+            // the two rows of a pair are two streams of the wave, or (SPLIT > 1) two neighbouring parts of it: the even
+            // part's first lane takes the odd part's sum from LPR lanes further on
             float second[R];
 #pragma unroll
-            for (int r = 0; r < R; r++) second[r] = HALF ? read_lane(sum[r], 32) : 0.0f;
-            if (lane == 0 && li0 < p.N) {
+            for (int r = 0; r < R; r++) {
+                second[r] = 0.0f;
+                if (HALF) second[r] = __shfl_xor(sum[r], LPR);
+            }
+            if (ll == 0 && (hf & 1) == 0 && li0 + hf < p.N) {
                 uint16_t* out = out_base;
                 if (loff != -1) out += (size_t)loff + (size_t)pos_now * p.N;
                 const int half = p.head_size >> 1;
                 const float2* cs_tab = p.rope + (size_t)pos_now * half;
 #pragma unroll
                 for (int r = 0; r < (HALF ? R : R - 1); r += (HALF ? 1 : 2)) {
-                    const int li = li0 + (HALF ? 2 * r : r);
+                    const int li = li0 + (HALF ? SPLIT * r + hf : r);
                     if (li < p.N) {
                         const int row = map_row<true>(li, p.head_size);
                         const float v0 = half_bits_to_float(float_to_half_bits(sum[r]));
@@ -223,7 +235,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
             if (loff != -1) out += (size_t)loff + (size_t)pos_now * p.N;
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const int row = li0 + (HALF ? 2 * r + hf : r);
+                const int row = li0 + (HALF ? SPLIT * r + hf : r);
                 if (row < p.N) {
                     float v;
                     if (KIND == KIND_FFN) {
@@ -373,9 +385,9 @@ int compute_units() {
     return cus;
 }
 
-template <int W, int R, int D, int KIND, bool ROPE, bool HALF = false>
+template <int W, int R, int D, int KIND, bool ROPE, int SPLIT = 1>
 int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
-    const int groups_total = div_up(p.N, W * R * (HALF ? 2 : 1));
+    const int groups_total = div_up(p.N, W * R * SPLIT);
     int gx = groups_total;
     // The norm-fused gate/up kernel stages (and normalises) x in every workgroup, and that work is what bounds it:
     // three 4-wave workgroups per compute unit walk the row groups between them (measured best at the 7B shape; the
@@ -388,7 +400,7 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
     if constexpr (KIND == KIND_SINGLE && !ROPE && R == 1 && W == 8) {  // (partial-sum input comes with K <= 8192: 8 waves)
         if (p.xpart) {
-            awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, false, true, HALF>, grid, dim3(W * 64), lds, p);
+            awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, false, true, SPLIT>, grid, dim3(W * 64), lds, p);
             return awq_check_launch(what);
         }
     }
@@ -397,17 +409,18 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
         return AWQ_ERR_ARG;
     }
     if (p.norm_w)
-        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, true, ROPE, false, HALF>, grid, dim3(W * 64), lds, p);
+        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, true, ROPE, false, SPLIT>, grid, dim3(W * 64), lds, p);
     else
-        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, ROPE, false, HALF>, grid, dim3(W * 64), lds, p);
+        awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, ROPE, false, SPLIT>, grid, dim3(W * 64), lds, p);
     return awq_check_launch(what);
 }
 
-// The half-wave forms: one row pair per wave (two gate/up pairs in the FFN form), `depth` passes of the pair in flight.
-template <int W, int KIND, bool ROPE>
-int dispatch_half(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, int depth) {
-    if (depth == 2) return launch<W, 1, 2, KIND, ROPE, true>(ctx, p, grid_y, what);
-    return launch<W, 1, 3, KIND, ROPE, true>(ctx, p, grid_y, what);
+// The split forms: one set of SPLIT rows per wave (SPLIT gate/up pairs in the FFN form), `depth` passes of the set in
+// flight.
+template <int W, int KIND, bool ROPE, int SPLIT>
+int dispatch_split(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, int depth) {
+    if (depth == 2) return launch<W, 1, 2, KIND, ROPE, SPLIT>(ctx, p, grid_y, what);
+    return launch<W, 1, 3, KIND, ROPE, SPLIT>(ctx, p, grid_y, what);
 }
 
 template <int W, int R, int KIND, bool ROPE>
@@ -462,8 +475,14 @@ int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan
     const int tail = p.C & 63;
     if (tail != 0 && tail <= 32 && plan.rows <= 2 && p.K <= 8192) {
         const int depth = KIND == KIND_QKV ? 2 : 3;
-        if (plan.waves == 4) return dispatch_half<4, KIND, ROPE>(ctx, p, grid_y, what, depth);
-        return dispatch_half<8, KIND, ROPE>(ctx, p, grid_y, what, depth);
+        // at most a quarter of a pass over (K = 6656): four rows to a wave pays for the QKV kernel (16.3 -> 15.6 us at the
+        // 33B shape); the O projection is unchanged by it and the gate/up kernel loses (21.8 -> 23.2: half as many row
+        // groups for its workgroups to walk)
+        if constexpr (KIND == KIND_QKV) {
+            if (tail <= 16) return dispatch_split<8, KIND, ROPE, 4>(ctx, p, grid_y, what, depth);
+        }
+        if (plan.waves == 4) return dispatch_split<4, KIND, ROPE, 2>(ctx, p, grid_y, what, depth);
+        return dispatch_split<8, KIND, ROPE, 2>(ctx, p, grid_y, what, depth);
     }
 #define AWQ_CASE(W_, R_) \
     if (plan.waves == W_ && plan.rows == R_) return dispatch_depth<W_, R_, KIND, ROPE>(ctx, p, grid_y, what, plan);
