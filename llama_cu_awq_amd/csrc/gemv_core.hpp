@@ -65,7 +65,7 @@ constexpr int XP = 2;
 // 4-wave workgroups carry four pieces per thread, so that vectors up to 8192 elements travel in registers whole (the late
 // fetch sits behind the staging barriers, one exposed round trip per 2048 elements: K = 5120 and 6656 at four waves),
 // 16-wave workgroups three (K = 17920).
-constexpr int pieces_for(int waves) { return waves <= 4 ? 4 : (waves >= 16 ? 3 : XP); }
+constexpr int pieces_for(int waves) { return waves <= 4 ? 4 : (waves >= 13 ? 3 : XP); }
 
 template <bool NORM, int NP = XP>
 struct XPieces {
@@ -115,7 +115,7 @@ __device__ __forceinline__ void load_parts(PartPieces& pr, const XArgs& p) {
 }
 
 template <int W>
-__device__ __forceinline__ void combine_x(XPieces<false>& xr, const PartPieces& pr, const XArgs& p) {
+__device__ __forceinline__ void combine_x(XPieces<false, pieces_for(W)>& xr, const PartPieces& pr, const XArgs& p) {
     constexpr int T = W * 64;
     const int n8 = p.K >> 3;
 #pragma unroll
@@ -224,11 +224,13 @@ __device__ __forceinline__ void stage_x(u32x4* xs, float* ca, const XArgs& p, fl
         // the correctly rounded divide, square root and reciprocal are ~60 instructions on a uniform value: one wave
         // computes them for the workgroup
         if (tid < 64) {
-            float r[W];
+            // pairwise tree over the waves' partial sums (wave counts that are no power of two: padded with zeros)
+            constexpr int WP = W <= 4 ? 4 : (W <= 8 ? 8 : 16);
+            float r[WP];
 #pragma unroll
-            for (int i = 0; i < W; i++) r[i] = red[i];
+            for (int i = 0; i < WP; i++) r[i] = i < W ? red[i] : 0.0f;
 #pragma unroll
-            for (int n = W; n > 1; n >>= 1)
+            for (int n = WP; n > 1; n >>= 1)
 #pragma unroll
                 for (int i = 0; i < n / 2; i++) r[i] = r[2 * i] + r[2 * i + 1];
             float t = r[0];

@@ -398,7 +398,7 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     }
     const dim3 grid(gx, grid_y);
     const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
-    if constexpr (KIND == KIND_SINGLE && !ROPE && R == 1 && W == 8) {  // (partial-sum input comes with K <= 8192: 8 waves)
+    if constexpr (KIND == KIND_SINGLE && !ROPE && R == 1 && (W == 8 || W == 10 || W == 13)) {  // (partial-sum input comes with K <= 8192)
         if (p.xpart) {
             awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, false, true, SPLIT>, grid, dim3(W * 64), lds, p);
             return awq_check_launch(what);
@@ -473,7 +473,34 @@ int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan
     // and even with three, tokens/s +3 %.  Rows above 8192 (K = 11008: 16 waves, or 8, at any depth) lose: two rows per
     // wave halve the workgroups of a matrix that has few rows to begin with.
     const int tail = p.C & 63;
-    if (tail != 0 && tail <= 32 && plan.rows <= 2 && p.K <= 8192) {
+    const bool split2 = tail != 0 && tail <= 32 && plan.rows <= 2 && p.K <= 8192;
+    if constexpr (KIND == KIND_SINGLE) {
+        // The workgroups of a single-matrix product are all resident at once, and the kernel takes as long as the
+        // compute unit that holds the most of them.  Workgroups of 10 or 13 waves are taken where they make the count a
+        // multiple of the compute units and the usual size does not (5120 rows: 256 workgroups of 10 two-row waves
+        // instead of 320 of 8, O projection from partial sums 7.8 -> 6.1 us, and 512 of 10 one-row waves instead of 640
+        // of 8, down projection 10.6 -> 9.9 us, at the 13B shape; 6656 rows: 13 waves).
+        if (plan.rows == 1 && (split2 || p.K > 8192)) {
+            const int cus = compute_units();
+            const int waves_total = div_up(p.N, split2 ? 2 : 1);
+            auto unevenness = [&](int w) {
+                const double per_cu = (double)div_up(waves_total, w) / cus;
+                return ceil(per_cu) / per_cu;
+            };
+            int best = plan.waves;
+            for (int w : {10, 13})
+                if (unevenness(w) < unevenness(best) - 0.15) best = w;
+            if (best == 10 || best == 13) {
+                if (split2) {
+                    if (best == 10) return dispatch_split<10, KIND, ROPE, 2>(ctx, p, grid_y, what, 3);
+                    return dispatch_split<13, KIND, ROPE, 2>(ctx, p, grid_y, what, 3);
+                }
+                if (best == 10) return dispatch_depth<10, 1, KIND, ROPE>(ctx, p, grid_y, what, plan);
+                return dispatch_depth<13, 1, KIND, ROPE>(ctx, p, grid_y, what, plan);
+            }
+        }
+    }
+    if (split2) {
         const int depth = KIND == KIND_QKV ? 2 : 3;
         // at most a quarter of a pass over (K = 6656): four rows to a wave pays for the QKV kernel (16.3 -> 15.6 us at the
         // 33B shape); the O projection is unchanged by it and the gate/up kernel loses (21.8 -> 23.2: half as many row
