@@ -28,10 +28,10 @@ HBM_PEAK = 8.0e12  # MI355X published HBM3E bandwidth, bytes/s
 # rocprofv3 summaries committed under profiles/, each named with its source.
 PROFILED = {
     # HBM bytes per launch of the norm-fused gate/up kernel at the 7B shape: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
-    "ffn_traffic_bytes": (47589376, "profiles/gemv_int4_ffn_7b_pmc.md"),
+    "ffn_traffic_bytes": (47585280, "profiles/gemv_int4_ffn_7b_pmc.md"),
     # rocprofv3 --kernel-trace average durations in the decode run, microseconds
-    "ffn_kernel_us": (10.38, "profiles/decode_7b_fused_kernel_trace.md"),
-    "gemv_4096_kernel_us": (4.42, "profiles/decode_7b_fused_kernel_trace.md"),
+    "ffn_kernel_us": (11.11, "profiles/decode_7b_fused_kernel_trace.md"),
+    "gemv_4096_kernel_us": (4.12, "profiles/decode_7b_fused_kernel_trace.md"),
 }
 
 
