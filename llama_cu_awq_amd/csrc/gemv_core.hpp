@@ -18,30 +18,35 @@ struct XArgs {
 };
 constexpr int kMaxParts = 4;
 
-// 2^-24 * sum over the 32 consecutive K elements of one chunk of (q - z) * x.
+// 2^-20 * sum over the 32 consecutive K elements of one chunk of (q - z) * x.
 //
-// w: 4 dwords of 8 nibbles.  xq[qi]: the 8 activations of dword qi as fp16 pairs
-// (x0,x4) (x1/16,x5/16) (x2,x6) (x3/16,x7/16).  A nibble masked out in place IS an fp16 number: with sign and
-// exponent bits zero, the bit pattern 0x000q is the denormal q * 2^-24 and 0x00q0 is 16q * 2^-24, both exact, and
-// v_dot2_f32_f16 takes denormal inputs at face value.  So each masked dword half multiplies its activation without
-// any offset to cancel: the products (at most 4 x 11 significant bits) are exact in fp32, and only the fp32
-// additions round, at the magnitude of the result itself (the reference adds fp32 products (q - z) * s * x the same
-// way, gpu_kernels.h:204-206).  The zero point comes in through the chunk's constant A = 2^-24 * sum x (computed
-// once when x is staged): the accumulator starts at -z * A.  The caller multiplies the result by 2^24 * scale.
+// w: 4 dwords of 8 nibbles.  xq[qi]: the 8 activations of dword qi as fp16 pairs (x0,x4) (x1,x5) (x2,x6) (x3,x7),
+// unscaled.  A nibble moved to bits 7..4 of an fp16 whose other bits are zero IS an fp16 number: the denormal
+// 16 q * 2^-24 = q * 2^-20, exact, and v_dot2_f32_f16 takes denormal inputs at face value.  So a shift and a mask are
+// the whole conversion, nothing has to be cancelled afterwards, and the activation enters the product as it is,
+// whatever its size (the reference multiplies (q - z) * s * x in fp32, gpu_kernels.h:203-207).
+//
+// Why bits 7..4 and not the nibble where it lies: v_dot2_f32_f16 forms both products exactly but adds them and the
+// accumulator inside a window of about 24 bits below the largest NOMINAL exponent of the three, truncating what falls
+// below.  A denormal's nominal exponent is that of the smallest normal number, so a nibble in bits 3..0 sits 6 to 10
+// bits below where the unit thinks it is and the accumulator loses that many bits at every step (measured at K = 4096:
+// 4.6 % of the fp16 outputs rounded differently from the exact result, against 0.1 % for the reference's sequential
+// fp32 sum and 0.07 % with every nibble in bits 7..4; bits 9..6 gain nothing more).  The price is two more shifts per
+// dword.  The zero point comes in through the chunk's constant A = 2^-20 * sum x (computed once when x is staged): the
+// accumulator starts at -z * A.  The caller multiplies the result by 2^20 * scale.
 __device__ __forceinline__ float chunk_dot(const u32x4 w, const float zf, const u32x4 (&xq)[4], const float A) {
     float acc = -zf * A;
 #pragma unroll
     for (int qi = 0; qi < 4; qi++) {
         const uint32_t d = w[qi];
-        const uint32_t d8 = d >> 8;
-        acc = dot2(d & 0x000F000Fu, xq[qi][0], acc);
+        acc = dot2((d << 4) & 0x00F000F0u, xq[qi][0], acc);
         acc = dot2(d & 0x00F000F0u, xq[qi][1], acc);
-        acc = dot2(d8 & 0x000F000Fu, xq[qi][2], acc);
-        acc = dot2(d8 & 0x00F000F0u, xq[qi][3], acc);
+        acc = dot2((d >> 4) & 0x00F000F0u, xq[qi][2], acc);
+        acc = dot2((d >> 8) & 0x00F000F0u, xq[qi][3], acc);
     }
     return acc;
 }
-constexpr float kChunkDotUnscale = 16777216.0f;  // 2^24
+constexpr float kChunkDotUnscale = 1048576.0f;  // 2^20
 
 // One 64-lane pass over the NS row streams of a wave: 16 bytes of packed weights per lane and stream, the zero-point
 // dword and the scale that cover them, and (residual form) the value the result is added to.
@@ -54,7 +59,7 @@ struct Stage {
 };
 
 // Staging of x (K halves) into LDS: xs[qi*C + c] holds the 8 activations of dword qi of chunk c as pairs
-// (x0,x4)(x1/16,x5/16)(x2,x6)(x3/16,x7/16), and ca[c] the chunk constant A described at chunk_dot.  Elements
+// (x0,x4)(x1,x5)(x2,x6)(x3,x7), and ca[c] the chunk constant A described at chunk_dot.  Elements
 // in [K, 32*C) are zero.  With NORM the vector is RMS-normalised on the way in with the reference's arithmetic
 // (gpu_kernels.h:72-105): o = half(x * (rsqrt(mean(x^2) + 1e-5) * w)).
 //
@@ -170,17 +175,14 @@ __device__ __forceinline__ void stage_piece(u32x4* xs, float* ca, const XArgs& p
         }
         if (store_norm && e < n8) reinterpret_cast<u32x4*>(p.norm_out)[e] = v;
     }
-    const h16x2 sixteenth = {(h16_t)0.0625f, (h16_t)0.0625f};
     // v holds halves h0..h7 as (h0,h1)(h2,h3)(h4,h5)(h6,h7) -> (h0,h4)(h1,h5)(h2,h6)(h3,h7)
     const h16x2 p0 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x05040100u));
-    const h16x2 p1 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x07060302u)) * sixteenth;
+    const h16x2 p1 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x07060302u));
     const h16x2 p2 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x05040100u));
-    const h16x2 p3 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x07060302u)) * sixteenth;
-    // fp32 sums of the stored halves: dot products against (1, 1)
+    const h16x2 p3 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x07060302u));
+    // fp32 sum of the 8 halves: dot products against (1, 1)
     const uint32_t ones = 0x3C003C00u;
-    const float even = dot2(as_u32(p0), ones, dot2(as_u32(p2), ones, 0.0f));
-    const float odd = dot2(as_u32(p1), ones, dot2(as_u32(p3), ones, 0.0f));
-    float a = fmaf(16.0f, odd, even);  // sum of the activations as the dot product sees them
+    float a = dot2(as_u32(p0), ones, dot2(as_u32(p1), ones, dot2(as_u32(p2), ones, dot2(as_u32(p3), ones, 0.0f))));
     // the 4 dword pieces of a chunk sit in 4 adjacent lanes
     a += dpp_mov<0xB1>(a);
     a += dpp_mov<0x4E>(a);

@@ -12,9 +12,9 @@
 // Each wave owns R consecutive rows (one gate/up pair in the fused FFN form) and walks them in passes of 64 x 16
 // bytes with D passes in flight.  Loads return in order, so a wave first requests its share of the activations,
 // then its first D passes of weights, and stages the activations while the weights are still on their way.
-// Nibbles are used in place as fp16 denormals (q * 2^-24: a mask is the whole conversion), products are accumulated
-// in fp32 by v_dot2_f32_f16, the zero point enters through a per-chunk constant, and the group scale (times 2^24) is
-// applied once per 32 elements.
+// Nibbles are used as fp16 denormals (a shift and a mask put q * 2^-20 into an fp16 lane: that is the whole conversion),
+// products are accumulated in fp32 by v_dot2_f32_f16, the zero point enters through a per-chunk constant, and the group
+// scale (times 2^20) is applied once per 32 elements.
 #include <math.h>
 
 #include "common.hpp"
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     // ---- consume cursor
     int cg = g_begin, cp = 0, cs = 0;
     auto finish_group = [&](const Stage<NS>& st) {
-        // chunk_dot works in units of 2^-24; with SPLIT > 1 every lane ends up with the sum of its own part of the wave
+        // chunk_dot works in units of 2^-20; with SPLIT > 1 every lane ends up with the sum of its own part of the wave
 #pragma unroll
         for (int i = 0; i < NS; i++) {
             float v = sum[i];
@@ -373,17 +373,9 @@ struct GemvPlan {
     int depth;   // stages in flight per wave (2, 3, 4)
 };
 
-int compute_units() {
-    static int cus = 0;
-    if (!cus) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
-    }
-    return cus;
-}
+// When set (by awq_gemv_geometry, on the calling thread), launch() reports the geometry it would launch with instead
+// of launching.
+thread_local awq_gemv_geometry_t* g_geometry_query = nullptr;
 
 template <int W, int R, int D, int KIND, bool ROPE, int SPLIT = 1>
 int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
@@ -393,8 +385,15 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     // three 4-wave workgroups per compute unit walk the row groups between them (measured best at the 7B shape; the
     // plain kernels are faster with one group per workgroup).
     if (p.norm_w && KIND == KIND_FFN) {
-        const int cus = compute_units();
+        const int cus = ctx->cus;
         if (gx > 3 * cus) gx = 3 * cus;
+    }
+    if (g_geometry_query) {
+        g_geometry_query->rows_per_group = W * R * SPLIT;
+        g_geometry_query->groups = groups_total;
+        g_geometry_query->grid_x = gx;
+        g_geometry_query->paired_rows = ROPE ? 1 : 0;
+        return AWQ_OK;
     }
     const dim3 grid(gx, grid_y);
     const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
@@ -464,7 +463,7 @@ int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan
         // with the most workgroups.  16-wave workgroups suit 4096 rows on 256 compute units (one each); 5120 rows are
         // 320 workgroups, two on a quarter of the compute units and one on the rest, and go better as 640 of 8 waves
         // (13B down projection 11.2 -> 10.7 us); 6656 rows are as uneven either way and keep 16 (measured).
-        const double per_cu16 = (double)div_up(p.N, 16) / compute_units(), per_cu8 = (double)div_up(p.N, 8) / compute_units();
+        const double per_cu16 = (double)div_up(p.N, 16) / ctx->cus, per_cu8 = (double)div_up(p.N, 8) / ctx->cus;
         if (ceil(per_cu8) / per_cu8 < ceil(per_cu16) / per_cu16 - 0.05) plan.waves = 8;
     }
     if (ROPE && plan.rows < 2) plan.rows = 2;  // a rotation pair lives in one wave
@@ -481,7 +480,7 @@ int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan
         // instead of 320 of 8, O projection from partial sums 7.8 -> 6.1 us, and 512 of 10 one-row waves instead of 640
         // of 8, down projection 10.6 -> 9.9 us, at the 13B shape; 6656 rows: 13 waves).
         if (plan.rows == 1 && (split2 || p.K > 8192)) {
-            const int cus = compute_units();
+            const int cus = ctx->cus;
             const int waves_total = div_up(p.N, split2 ? 2 : 1);
             auto unevenness = [&](int w) {
                 const double per_cu = (double)div_up(waves_total, w) / cus;
@@ -590,6 +589,28 @@ int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qwe
     p.norm_w = norm_w;
     p.norm_out = norm_out;
     return dispatch<KIND_FFN, false>(ctx, p, 1, "ffn_matvec_silu", plan_for(K, 1));
+}
+
+// Internal: the launch geometry the dispatcher picks for a product (nothing is launched).  kind: 0 single matrix
+// (norm: RMSNorm fused; parts: input as partial sums), 2 gate/up.  Row group g (rows_per_group consecutive rows, of both
+// matrices in the gate/up form) is read by workgroup g % grid_x.
+int awq_gemv_geometry(awq_ctx* ctx, int kind, int K, int N, int norm, int parts, awq_gemv_geometry_t* out) {
+    static const uint16_t dummy = 0;
+    GemvParams p;
+    fill_common(p, &dummy, K, N);
+    if (norm) p.norm_w = &dummy;
+    if (parts) {
+        p.xpart = reinterpret_cast<const float*>(&dummy);
+        p.xparts = parts;
+    }
+    g_geometry_query = out;
+    int r;
+    if (kind == 2)
+        r = dispatch<KIND_FFN, false>(ctx, p, 1, "geometry", plan_for(K, 1));
+    else
+        r = dispatch<KIND_SINGLE, false>(ctx, p, 1, "geometry", plan_for(K, 1));
+    g_geometry_query = nullptr;
+    return r;
 }
 
 extern "C" {

@@ -61,8 +61,15 @@ static int ctx_init(int device, hipStream_t stream, bool owns, awq_ctx** out) {
         if (owns) (void)hipStreamDestroy(stream);
         return r;
     }
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) {
+        if (owns) (void)hipStreamDestroy(stream);
+        awq_set_error("cannot read the compute-unit count of device %d", device);
+        return AWQ_ERR_HIP;
+    }
     awq_ctx* c = new awq_ctx();
     c->device = device;
+    c->cus = cus;
     c->stream = stream;
     c->owns_stream = owns;
     c->probe = nullptr;

@@ -149,7 +149,7 @@ __device__ __forceinline__ float chunk_dot(const u32x4 w, const float zf, const 
         acc0 = dot2((d8 & 0x000F000Fu) | magic, xq[qi][2], acc0);
         acc1 = dot2((d8 & 0x00F000F0u) | magic, xq[qi][3], acc1);
     }
-    return acc0 + acc1;
+    return fmaf(acc1, 0.0625f, acc0);  // the high nibbles enter 16 times too large; the activations are never scaled
 }
 
 // Consume one landed unit: returns this lane's contribution to the row's dot product.
@@ -230,7 +230,6 @@ __device__ void stage_input(const Args& a, PhasePtr P, int ht, int lane, int hw,
             ss = 1.0f / sqrtf(ss);
         }
         const u32x4* wg = reinterpret_cast<const u32x4*>(P->norm_w);
-        const h16x2 sixteenth = {(h16_t)0.0625f, (h16_t)0.0625f};
         const int total = P->kind == KIND_CLS ? n8 : P->C * 4;
 #pragma unroll
         for (int i = 0; i < MAXP; i++) {
@@ -251,15 +250,16 @@ __device__ void stage_input(const Args& a, PhasePtr P, int ht, int lane, int hw,
             if (P->kind == KIND_CLS) {
                 if (e < total) xs[e] = v;
             } else {
-                // (h0,h1)(h2,h3)(h4,h5)(h6,h7) -> (h0,h4)(h1/16,h5/16)(h2,h6)(h3/16,h7/16)
+                // (h0,h1)(h2,h3)(h4,h5)(h6,h7) -> (h0,h4)(h1,h5)(h2,h6)(h3,h7)
                 const h16x2 p0 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x05040100u));
-                const h16x2 p1 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x07060302u)) * sixteenth;
+                const h16x2 p1 = as_h2(__builtin_amdgcn_perm(v[2], v[0], 0x07060302u));
                 const h16x2 p2 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x05040100u));
-                const h16x2 p3 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x07060302u)) * sixteenth;
+                const h16x2 p3 = as_h2(__builtin_amdgcn_perm(v[3], v[1], 0x07060302u));
                 const float even = ((float)p0[0] + (float)p0[1]) + ((float)p2[0] + (float)p2[1]);
                 const float odd = ((float)p1[0] + (float)p1[1]) + ((float)p3[0] + (float)p3[1]);
-                float sa = fmaf(16.0f, odd, even);
-                float sb = even + odd;
+                // even positions meet 1024 + q, odd positions (1024 + 16 q) / 16 = 64 + q
+                float sa = even + odd;
+                float sb = fmaf(0.0625f, odd, even);
                 sa += dpp_mov<0xB1>(sa);
                 sa += dpp_mov<0x4E>(sa);
                 sb += dpp_mov<0xB1>(sb);

@@ -65,34 +65,65 @@ def _oracle_record(o, n_prompt, steps, first_pos=0):
 def _conditioning(o, ref, n_prompt, first_pos=0):
     """How far the oracle's logits move when its matrix-vector sums are rounded once from double precision instead
     of being added in the reference's fp32 order: the same passes again from the oracle's state before `ref` was
-    recorded (the caller restores that state), kept on ref's tokens.  Returns the per-pass rel-L2 distances."""
+    recorded (the caller restores that state), kept on ref's tokens.  Returns the per-pass rel-L2 distances and the
+    logits of the exactly summed passes."""
     vocab = o.config["vocab_size"]
-    dist = []
+    dist, exact = [], []
     oracle.set_exact_sums(True)
     try:
         for i, (want_logits, want_tok) in enumerate(ref):
             gen = i >= n_prompt - 1
             o.forward(gen)
             pos = first_pos + i
-            dist.append(rel_l2(f16(o.buffer("logits", vocab)), want_logits))
+            exact.append(f16(o.buffer("logits", vocab)).copy())
+            dist.append(rel_l2(exact[-1], want_logits))
             if gen and o.tokens(pos + 2)[pos + 1] != want_tok:
                 o.set_pos(pos + 1, int(want_tok))
     finally:
         oracle.set_exact_sums(False)
-    return dist
+    return dist, exact
+
+
+# How much farther from the exactly summed logits than the reference's own fp32 order a GPU run may be.  Any fp32
+# summation order is one sample of the same rounding noise, amplified through 32 to 60 layers of near-argmax softmax by
+# a factor that differs from pass to pass; and the passes of a run share their history (each reads the KV rows its
+# predecessors wrote), so a run is one sample of a trajectory, not 16 or 48 independent ones.  Measured over the five
+# scenarios below the ratio GPU / reference order of the median distance is 0.99 .. 1.54 and of the worst pass
+# 0.89 .. 2.05.  The comparison is therefore between the two runs' distributions over the passes: median and mean
+# within EXACT_FACTOR, the worst pass within EXACT_WORST of the reference order's worst.  Position 0 (no attention,
+# nothing amplified, no history) is compared on its own by the callers that start there, and the arithmetic of a
+# single product is held much tighter in tests/test_gpu_ops.py (how many outputs round differently from the exact sum).
+EXACT_FACTOR = 2.0
+EXACT_WORST = 2.5
+
+
+def _check_against_exact(rec, exact, dist, what):
+    """The comparison the arithmetic fixes, whatever the model's conditioning: the GPU's logits are no farther from the
+    exactly summed ones (every matrix-vector sum rounded once from double precision, same token history) than the
+    reference's fp32 summation order is."""
+    g = [rel_l2(logits, ex) for (logits, _), ex in zip(rec, exact)]
+    med_g, med_d = float(np.median(g)), float(np.median(dist))
+    print(f"{what}: distance from exactly summed logits, GPU / the reference's fp32 order, per pass:")
+    print("  " + " ".join(f"{a:.4f}/{b:.4f}" for a, b in zip(g, dist)))
+    print(f"  GPU worst {max(g):.4g} mean {np.mean(g):.4g} median {med_g:.4g}; reference order worst {max(dist):.4g} "
+          f"mean {np.mean(dist):.4g} median {med_d:.4g}")
+    assert med_g <= EXACT_FACTOR * med_d, (med_g, med_d)
+    assert float(np.mean(g)) <= EXACT_FACTOR * float(np.mean(dist)), (float(np.mean(g)), float(np.mean(dist)))
+    assert max(g) <= EXACT_WORST * max(dist), (max(g), max(dist))
+    return g
 
 
 def _bars(dist):
     """(per-pass bar, median bar) for GPU-vs-oracle logits from the oracle's own sensitivity `dist`: two
     implementations that each differ from the exactly rounded sums by about that much differ from each other by more
     (independent differences, different exponentials), hence the factors; never below the benchmark's 1e-2."""
-    return max(1e-2, 6 * max(dist)), max(1e-2, 3 * float(np.median(dist)))
+    return max(1e-2, 4 * max(dist)), max(1e-2, 2.5 * float(np.median(dist)))
 
 
 def _gpu_record(t, n_prompt, steps, use_graph, mode, first_pos=0, ref=None, bar=1e-2):
     """The same passes on the GPU (synchronise, launch, read back: the reference loop).  With `ref` (a record of the
-    oracle or of another GPU run) every pass is checked against it: logits within rel-L2 1e-2 and the same greedy
-    token.
+    oracle or of another GPU run) every pass is compared with it: the rel-L2 distance of the logits is returned for the
+    caller to hold against its bar, and the greedy token must be the same or a tie as defined below.
 
     Random weights put the largest of 32000 fp16 logits a few fp16 steps apart, and exact ties are common (the
     oracle's own 7B run has five among its first 32 generated tokens; it breaks them by lowest index), so two correct
@@ -162,11 +193,12 @@ def _bars_7b(model_7b):
         ref = _oracle_record(o, n_prompt, steps)
         assert all(np.isfinite(l.astype(np.float32)).all() for l, _ in ref)
         o.reset(prompt)
-        dist = _conditioning(o, ref, n_prompt)
+        dist, exact = _conditioning(o, ref, n_prompt)
         print(f"oracle, reference summation order vs sums rounded once: logits rel-L2 worst {max(dist):.3g}, median {np.median(dist):.3g}")
         assert max(dist) > 1e-2  # the reason for the derived bar; if this stops holding, hold the run to 1e-2 outright
         shared["bars"] = _bars(dist)
         shared["ref"] = (prompt, ref)
+        shared["exact"] = (dist, exact)
     return shared["bars"]
 
 
@@ -179,7 +211,9 @@ def test_7b_prompt_then_32_greedy_steps(model_7b):
     t.reset(prompt)
     rec, errs, ties = _gpu_record(t, n_prompt, steps, True, A.SCHEDULE_FUSED, ref=ref, bar=shared["bars"][0])
     _check(errs, shared["bars"])
-    assert errs[0] <= 1e-2  # position 0 has no attention to amplify anything
+    g = _check_against_exact(rec, shared["exact"][1], shared["exact"][0], "7B shape, 16 prompt + 32 generated tokens")
+    assert errs[0] <= 1e-2  # position 0 has no attention to amplify anything:
+    assert g[0] <= 1.5 * shared["exact"][0][0]  # there the single pass is comparable
     assert [t.token(i) for i in range(n_prompt)] == prompt
     assert [tok for _, tok in rec] == [tok for _, tok in ref]
     assert ties <= 10, ties  # the oracle's own 32 steps have 5 pairs of top logits within 2 fp16 steps, 3 of them exact ties
@@ -198,11 +232,14 @@ def test_7b_decode_across_sequence_length_bins(model_7b, start):
     _prefill_kv_both(t, o, cfg, seed=start, upto=start)
     o.set_pos(start, tok0)
     ref = _oracle_record(o, 1, steps, first_pos=start)
+    o.set_pos(start, tok0)
+    dist, exact = _conditioning(o, ref, 1, first_pos=start)
     for use_graph in (False, True):
         t.set_pos(start, tok0)  # the rows from `start` on are rewritten by the passes themselves
         rec, errs, ties = _gpu_record(t, 1, steps, use_graph, A.SCHEDULE_FUSED, first_pos=start, ref=ref, bar=bars[0])
         assert t.pos == start + steps
         _check(errs, bars)
+        _check_against_exact(rec, exact, dist, f"7B shape, 16 passes from position {start}")
         assert ties <= 4, ties
 
 
@@ -356,12 +393,13 @@ def test_13b_decode_from_kv_prefilled_to_1536(ctx):
         ref = _oracle_record(o, 1, steps, first_pos=start)
         assert all(np.isfinite(l.astype(np.float32)).all() for l, _ in ref)
         o.set_pos(start, tok0)
-        dist = _conditioning(o, ref, 1, first_pos=start)
+        dist, exact = _conditioning(o, ref, 1, first_pos=start)
         print(f"oracle, reference summation order vs sums rounded once: logits rel-L2 worst {max(dist):.3g}, median {np.median(dist):.3g}")
         for use_graph in (False, True):
             t.set_pos(start, tok0)  # the rows from `start` on are rewritten by the passes themselves
-            _, errs, ties = _gpu_record(t, 1, steps, use_graph, A.SCHEDULE_FUSED, first_pos=start, ref=ref, bar=_bars(dist)[0])
+            rec, errs, ties = _gpu_record(t, 1, steps, use_graph, A.SCHEDULE_FUSED, first_pos=start, ref=ref, bar=_bars(dist)[0])
             _check(errs, _bars(dist))
+            _check_against_exact(rec, exact, dist, "13B shape from a cache pre-filled to 1536")
             assert ties <= 2, ties
     finally:
         t.close()
@@ -412,7 +450,7 @@ def test_33b_full_model_schedules_agree_and_stay_finite(ctx):
         o.reset(prompt)
         ref = _oracle_record(o, n_prompt, n_prompt + 3)
         o.reset(prompt)
-        dist = _conditioning(o, ref, n_prompt)
+        dist, exact = _conditioning(o, ref, n_prompt)
         print(f"oracle, reference summation order vs sums rounded once: logits rel-L2 worst {max(dist):.3g}, median {np.median(dist):.3g}")
         bars = _bars(dist)
         for graph in (False, True):
@@ -421,8 +459,9 @@ def test_33b_full_model_schedules_agree_and_stay_finite(ctx):
             _check(errs, bars)
             assert ties <= 4, ties
         t.reset(prompt)
-        _, errs, _ = _gpu_record(t, n_prompt, n_prompt + 3, True, A.SCHEDULE_FUSED, ref=ref, bar=bars[0])
+        rec, errs, _ = _gpu_record(t, n_prompt, n_prompt + 3, True, A.SCHEDULE_FUSED, ref=ref, bar=bars[0])
         _check(errs, bars)
+        _check_against_exact(rec, exact, dist, "33B shape, all 60 layers, half the scale range")
     finally:
         t.close()
         o.close()
