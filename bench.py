@@ -6,7 +6,8 @@ random prompt as warm-up and times exactly 256 decode steps; weights are random 
 real layout and distributions, resident in HBM before the timed region starts.
 
 Prints ONE JSON line: tokens/s (`value`) of the run the flags ask for; `config1`, the benchmark's own run (16-token
-prompt + 256 decode steps from position 0) whatever the flags were; the roofline of the dominant kernel as the timed
+prompt + 256 decode steps from position 0) whatever the flags were; `config2` and `config3`, short runs of the 13B shape
+from a KV cache pre-filled to position 1536 and of the 33B shape; the roofline of the dominant kernel as the timed
 schedule launches it (RMSNorm-fused gate/up int4 matrix-vector product, timed live with HIP events over the 32
 layers' distinct weights); `config0`, the single 4096 x 4096 product back to back on one stream and dealt over 2 and 4
 plain streams; the 512-token prefill; and the CPU oracle timed on a bounded sample of the same workload.
@@ -24,15 +25,41 @@ if ROOT not in sys.path:
 
 HBM_PEAK = 8.0e12  # MI355X published HBM3E bandwidth, bytes/s
 
-# Figures that cannot be measured inside this process (hardware counters, profiler durations): read from the
-# rocprofv3 summaries committed under profiles/, each named with its source.
-PROFILED = {
-    # HBM bytes per launch of the norm-fused gate/up kernel at the 7B shape: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0
-    "ffn_traffic_bytes": (47585280, "profiles/gemv_int4_ffn_7b_pmc.md"),
-    # rocprofv3 --kernel-trace average durations in the decode run, microseconds
-    "ffn_kernel_us": (11.11, "profiles/decode_7b_fused_kernel_trace.md"),
-    "gemv_4096_kernel_us": (4.12, "profiles/decode_7b_fused_kernel_trace.md"),
-}
+# Figures that cannot be measured inside this process (hardware counters, profiler durations) are read, at run time,
+# from the rocprofv3 summaries committed under profiles/: the table rows of the kernels named here.
+TRACE_MD = "profiles/decode_7b_fused_kernel_trace.md"
+PMC_MD = "profiles/gemv_int4_ffn_7b_pmc.md"
+FFN_KERNEL = "gemv_int4_kernel<4, 1, 2, 2, true, false, false, 1>"  # norm-fused gate/up, the launch of the fused schedule
+GEMV_4096_KERNEL = "gemv_int4_kernel<8, 1, 2, 0, false, false, false, 1>"  # O projection and the 4096 x 4096 loops
+COPY_ROW = "__amd_rocclr_copyBuffer, 256 MiB"
+
+
+def _table_row(path, starts_with):
+    """Cells (stripped) of the first markdown table row of `path` whose first cell starts with `starts_with`."""
+    with open(os.path.join(ROOT, path)) as f:
+        for line in f:
+            if line.startswith("|"):
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if cells and cells[0].startswith(starts_with):
+                    return cells
+    raise KeyError(f"{path}: no table row for {starts_with}")
+
+
+def profiled_figures():
+    """rocprofv3 figures of the 7B-shape kernels from the committed summaries: average kernel durations (us) of the
+    kernel trace, and the HBM bytes per launch of the roofline kernel from the FETCH_SIZE / WRITE_SIZE counters (KiB per
+    dispatch), each scaled by what the same counter reads for a 256 MiB device copy."""
+    num = lambda c: float(c.replace(",", ""))
+    ffn_us = num(_table_row(TRACE_MD, FFN_KERNEL)[2])
+    gemv_us = num(_table_row(TRACE_MD, GEMV_4096_KERNEL)[2])
+    copy = _table_row(PMC_MD, COPY_ROW)
+    ffn = _table_row(PMC_MD, FFN_KERNEL)
+    fetch_scale = 262144.0 / num(copy[2])  # KiB actually read by the copy / KiB the counter shows for it
+    write_scale = 262144.0 / num(copy[3])
+    fetch_scale, write_scale = round(fetch_scale, 1), round(write_scale, 1)  # the factors as the summary states them
+    traffic = int(round((num(ffn[2]) * fetch_scale + num(ffn[3]) * write_scale) * 1024))
+    return {"ffn_kernel_us": ffn_us, "gemv_4096_kernel_us": gemv_us, "ffn_traffic_bytes": traffic,
+            "fetch_scale": fetch_scale, "write_scale": write_scale}
 
 
 def qweight_bytes(K, N):
@@ -59,6 +86,7 @@ def main():
     ap.add_argument("--cpu-tokens", type=int, default=12, help="tokens of the same model timed on the CPU oracle (0 = skip)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--prefill", type=int, default=512, help="also time a batched prefill of this many prompt tokens (0 = skip)")
+    ap.add_argument("--no-extra-configs", action="store_true", help="skip the 13B-shape and 33B-shape runs that a 7B run appends")
     ap.add_argument("--only-kernels", action="store_true", help="skip the decode loop: run only the per-kernel loops and a 256 MiB device copy (for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -88,18 +116,23 @@ def main():
     vocab = cfg["vocab_size"]
     kv_dim = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"]
     prompt = synth.prompt_tokens(args.seed, n_prompt, vocab)
-    if args.start_pos:
-        # KV cache pre-filled with N(0,1) below start_pos (long-context configuration)
-        for name in ("key_cache", "value_cache"):
-            buf = model.buffer(name, cfg["n_layers"] * cfg["seq_len"] * kv_dim * 2)
-            for l in range(cfg["n_layers"]):
-                vals = synth.normal_f16(synth.stream_key(args.seed, name, l), args.start_pos * kv_dim)
-                buf.write(vals, offset_bytes=l * cfg["seq_len"] * kv_dim * 2)
 
-    def run_decode(n_prompt, n_steps, start_pos=0):
+    def fill_kv(model, cfg, upto):
+        """KV cache pre-filled with N(0,1) below position `upto` (the long-context configuration)."""
+        kvd = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"]
+        for name in ("key_cache", "value_cache"):
+            buf = model.buffer(name, cfg["n_layers"] * cfg["seq_len"] * kvd * 2)
+            for l in range(cfg["n_layers"]):
+                vals = synth.normal_f16(synth.stream_key(args.seed, name, l), upto * kvd)
+                buf.write(vals, offset_bytes=l * cfg["seq_len"] * kvd * 2)
+
+    if args.start_pos:
+        fill_kv(model, cfg, args.start_pos)
+
+    def run_decode(model, cfg, n_prompt, n_steps, start_pos=0):
         """Prompt as warm-up, then n_steps timed decode steps with the reference's synchronise-then-launch loop
         (llama2_q4.cu:713).  Every recorded launch sequence the run will replay is recorded before the clock starts."""
-        toks = synth.prompt_tokens(args.seed, n_prompt, vocab)
+        toks = synth.prompt_tokens(args.seed, n_prompt, cfg["vocab_size"])
         model.reset(toks)
         if start_pos:
             model.set_pos(start_pos, toks[0])
@@ -136,7 +169,7 @@ def main():
             check(lib.awq_memcpy_d2d_async(ctx.h, dst.ptr, src.ptr, nbytes))
         ctx.sync()
         args.steps, n_prompt, total = 1, 1, 2
-    wall, gpu_ms, gen = run_decode(n_prompt, args.steps, args.start_pos)
+    wall, gpu_ms, gen = run_decode(model, cfg, n_prompt, args.steps, args.start_pos)
     tok_s = args.steps / wall
 
     wbytes = weight_bytes_per_token(cfg)
@@ -198,9 +231,11 @@ def main():
         "bytes_per_product": gemv_bytes,
         "one_stream_back_to_back": {"us_per_product": round(gemv_us, 3), "gbps": round(gemv_gbps, 1), "frac": round(gemv_gbps * 1e9 / HBM_PEAK, 4)},
     }
-    if (dim, hid) == (4096, 11008):
-        us, src = PROFILED["gemv_4096_kernel_us"]
-        config0["rocprof_kernel_duration"] = {"us_per_product": us, "gbps": round(gemv_bytes / us / 1e3, 1), "frac": round(gemv_bytes / us / 1e3 / 8000.0, 4), "source": src}
+    is_7b = (dim, hid) == (4096, 11008)
+    prof = profiled_figures() if is_7b else None
+    if is_7b:
+        us = prof["gemv_4096_kernel_us"]
+        config0["rocprof_kernel_duration"] = {"us_per_product": us, "gbps": round(gemv_bytes / us / 1e3, 1), "frac": round(gemv_bytes / us / 1e3 / 8000.0, 4), "source": TRACE_MD}
     # the same product through the C-ABI from one host thread per stream: 1, 2 and 4 plain streams over 64 distinct
     # matrices (558 MB), so that the fixed cost of a dependent launch overlaps the streaming of the other streams
     tool = os.path.join(ROOT, "llama_cu_awq_amd", "bin", "gemv_bench")
@@ -220,7 +255,7 @@ def main():
         if (n_prompt, args.steps, args.start_pos) == (16, 256, 0):
             c_wall, c_gpu_ms, c_gen = wall, gpu_ms, gen
         else:
-            c_wall, c_gpu_ms, c_gen = run_decode(16, 256, 0)
+            c_wall, c_gpu_ms, c_gen = run_decode(model, cfg, 16, 256, 0)
         config1 = {
             "workload": "16-token prompt then 256 decode steps from position 0",
             "tok_per_s": round(256 / c_wall, 2),
@@ -278,6 +313,40 @@ def main():
         }
         o.close()
 
+    # ---- configurations 2 and 3 (13B shape from a cache pre-filled to 1536; 33B shape), compact, after everything that
+    # needs the 7B model.  The 33B image takes half the benchmark's scale range: with the full range the residual stream
+    # of a 60-layer model leaves fp16 range (in the oracle as on the GPU) and its tokens would mean nothing.
+    extra = {}
+    if args.config == "7b" and not args.only_kernels and not args.no_extra_configs:
+        model.close()
+        model = None
+        del image
+        for key, name, start, steps, scale in (("config2", "13b", 1536, 64, 1.0), ("config3", "33b", 0, 32, 0.5)):
+            xcfg = {"13b": synth.CONFIG_13B, "33b": synth.CONFIG_33B}[name]
+            t0 = time.time()
+            ximg = synth.make_model_image(xcfg, seed=args.seed, threads=min(16, os.cpu_count() or 8), scale_mult=scale)
+            xm = A.Transformer(ctx, image=ximg)
+            print(f"[bench] {name} image {ximg.nbytes / 1e9:.2f} GB generated and uploaded in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+            del ximg
+            if start:
+                fill_kv(xm, xcfg, start)
+            x_wall, x_gpu_ms, x_gen = run_decode(xm, xcfg, 4, steps, start)
+            xw = weight_bytes_per_token(xcfg)
+            xkv = 2 * xcfg["n_layers"] * (xcfg["dim"] * xcfg["n_kv_heads"] // xcfg["n_heads"]) * 2 * (start + 4 + (steps + 1) / 2.0)
+            x_tok_s = steps / x_wall
+            extra[key] = {
+                "workload": f"llama-{name}-shape: 4-token prompt then {steps} decode steps from position {start}" + (" (KV cache pre-filled with N(0,1))" if start else "") + (f", scale range x {scale}" if scale != 1.0 else ""),
+                "tok_per_s": round(x_tok_s, 2),
+                "ms_per_step": round(x_wall * 1e3 / steps, 4),
+                "gpu_ms_per_step": round(x_gpu_ms / steps, 4),
+                "weight_bytes_per_token": xw,
+                "avg_kv_bytes_per_token": int(xkv),
+                "frac_of_weight_roofline": round(x_tok_s / (HBM_PEAK / xw), 4),
+                "frac_of_weight_plus_kv_roofline": round(x_tok_s / (HBM_PEAK / (xw + xkv)), 4),
+                "first_tokens": x_gen,
+            }
+            xm.close()
+
     out = {
         "metric": "decode tok/s bs=1 @7B shape; int4 GEMV HBM GB/s vs ~8 TB/s peak",
         "value": round(tok_s, 2),
@@ -303,17 +372,21 @@ def main():
             "achieved": round(ffn_gbps, 1),
             "peak": HBM_PEAK / 1e9,
             "unit": "GB/s",
+            # achieved and frac follow from ONE measurement: this process's HIP events around the launches in place
+            # (us_per_launch below); the committed rocprofv3 trace of the same command is carried beside it as frac_rocprof
             "frac": round(ffn_gbps * 1e9 / HBM_PEAK, 4),
+            "frac_source": "HIP events in this run (us_per_launch)",
+            "frac_rocprof": round(ffn_bytes / prof["ffn_kernel_us"] / 1e3 / (HBM_PEAK / 1e9), 4) if is_7b else None,
             # HBM bytes per launch cannot be counted from inside the run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this
             # kernel at the 7B shape, from the committed summary
-            "traffic": PROFILED["ffn_traffic_bytes"][0] if (dim, hid) == (4096, 11008) else None,
-            "traffic_source": PROFILED["ffn_traffic_bytes"][1] if (dim, hid) == (4096, 11008) else None,
+            "traffic": prof["ffn_traffic_bytes"] if is_7b else None,
+            "traffic_source": PMC_MD if is_7b else None,
             "bytes_per_launch": ffn_bytes,
             "us_per_launch": round(ffn_us, 3),
             "how_timed": "start/stop HIP events attached to each of the %d gate/up launches (kernel start to kernel end) in 4 eager passes of the fused schedule at position %d, on the context's stream" % (cfg["n_layers"], mid),
             "isolated_loop_us_per_launch": round(ffn_loop_us, 3),
-            "rocprof_us_per_launch": PROFILED["ffn_kernel_us"][0] if (dim, hid) == (4096, 11008) else None,
-            "rocprof_source": PROFILED["ffn_kernel_us"][1] if (dim, hid) == (4096, 11008) else None,
+            "rocprof_us_per_launch": prof["ffn_kernel_us"] if is_7b else None,
+            "rocprof_source": TRACE_MD if is_7b else None,
             "plain_form_us_per_launch": round(ffn_plain_us, 3),
         },
         "cpu_baseline": cpu,
@@ -330,8 +403,10 @@ def main():
         "config0": config0,
         "config1": config1,
     }
+    out.update(extra)
     print(json.dumps(out), flush=True)
-    model.close()
+    if model is not None:
+        model.close()
     ctx.close()
 
 

@@ -75,6 +75,9 @@ int awq_memcpy_h2d_async(awq_ctx* ctx, void* dst, const void* src, size_t bytes)
 int awq_memcpy_h2d(awq_ctx* ctx, void* dst, const void* src, size_t bytes); /* blocking */
 int awq_memcpy_d2h(awq_ctx* ctx, void* dst, const void* src, size_t bytes); /* blocking, ordered after the stream */
 int awq_memcpy_d2d_async(awq_ctx* ctx, void* dst, const void* src, size_t bytes);
+/* (hipMemsetAsync on the context's stream.  Not for a stream that is being captured into a graph: memset nodes have
+ * given wrong results on replays after the first on this platform; inside a capture clear memory with a kernel, as the
+ * library's own recorded sequences do.) */
 int awq_memset_async(awq_ctx* ctx, void* dst, int value, size_t bytes);
 
 /* ---- timing on the context's stream (cudaEvent pair, llama2_q4.cu:545-550, 592-600). */
@@ -214,10 +217,12 @@ int awq_transformer_set_pos(awq_transformer* t, int pos, int token);
  * use_graph != 0 replays a recorded launch sequence keyed by sequence-length bin (the USE_CUDA_GRAPHS path,
  * llama2_q4.cu:553-575); 0 launches eagerly.  mode selects the schedule: AWQ_SCHEDULE_REFERENCE issues the
  * reference's op sequence one launcher at a time; AWQ_SCHEDULE_FUSED merges RMSNorm into the consuming
- * matrix-vector kernels (same rounding points); AWQ_SCHEDULE_PERSISTENT runs the whole token, sampler included,
- * as ONE launch of a persistent kernel (one workgroup per CU, grid barriers between the steps, weights prefetched
- * across steps); it ignores use_graph and returns AWQ_ERR_SHAPE for models whose shape its work split cannot take
- * (the other two schedules run every model). */
+ * matrix-vector kernels (same rounding points) and is the one to use.
+ * AWQ_SCHEDULE_PERSISTENT is EXPERIMENTAL and about 2.3x SLOWER than FUSED (379 against 869 tokens/s at the 7B shape):
+ * the whole token, sampler included, as ONE launch of a persistent kernel (one workgroup per CU, grid barriers between
+ * the steps, weights prefetched across steps).  It produces the same tokens, ignores use_graph and returns
+ * AWQ_ERR_SHAPE for models whose shape its work split cannot take (the other two schedules run every model).  Kept
+ * as a record of what a grid barrier costs on this part (as much as a kernel boundary); not tuned further. */
 #define AWQ_SCHEDULE_REFERENCE 0
 #define AWQ_SCHEDULE_FUSED 1
 #define AWQ_SCHEDULE_PERSISTENT 2

@@ -34,44 +34,6 @@ struct awq_ctx {
     size_t gemm_counter_count;
 };
 
-// Launch geometry of an int4 matrix-vector product as the dispatcher picks it (awq_gemv_geometry).
-struct awq_gemv_geometry_t {
-    int rows_per_group;  // consecutive rows (gate/up form: rows of each of the two matrices) that one workgroup takes at a time
-    int groups;          // row groups in all
-    int grid_x;          // workgroups along x; group g is read by workgroup g % grid_x
-    int paired_rows;     // rows are dealt in rotation pairs (i, i + head/2): groups are not runs of consecutive rows
-};
-
-// What a kernel with idle workgroups may pull into the L2 caches for the launch that follows it.  L2 is per XCD and
-// keeps clean lines across a kernel boundary (measured: a region of up to 32 MiB re-read by the next launch from the
-// same XCDs streams at 14 TB/s with 0.28 us latency, against 7.5 TB/s and 0.93 us from HBM), and workgroup i of a
-// launch runs on XCD i % 8, so a line helps only in the L2 of the XCD whose workgroup will read it.  A segment is a
-// run of `nblocks` blocks of `block_bytes`; block j belongs to XCD j % 8.  nblocks == 0: the whole range
-// [base, base + block_bytes) is wanted on every XCD.
-struct awq_prefetch_seg {
-    const char* base;
-    uint32_t block_bytes;
-    uint32_t nblocks;
-    uint32_t lines_per_block;  // 128-byte lines a block can touch (one more than its size when it starts off a line)
-    uint32_t inv_lines;        // floor(2^32 / lines_per_block) + 1: i / lines_per_block == mulhi(i, inv_lines) for i < 2^20
-};
-static inline awq_prefetch_seg awq_make_prefetch_seg(const void* base, size_t block_bytes, uint32_t nblocks) {
-    awq_prefetch_seg sg;
-    sg.base = reinterpret_cast<const char*>(base);
-    sg.block_bytes = (uint32_t)block_bytes;
-    sg.nblocks = nblocks;
-    const uintptr_t b = reinterpret_cast<uintptr_t>(base);
-    sg.lines_per_block = nblocks ? (uint32_t)((block_bytes + 127) / 128 + 1) : (uint32_t)(((b + block_bytes - 1) >> 7) - (b >> 7) + 1);
-    sg.inv_lines = (uint32_t)(0x100000000ull / sg.lines_per_block) + 1;
-    return sg;
-}
-constexpr int kPrefetchSegs = 12;
-constexpr size_t kPrefetchBudgetBytes = (size_t)24 << 20;  // of the 32 MiB of L2, what one launch may ask for
-struct awq_prefetch_plan {
-    awq_prefetch_seg seg[kPrefetchSegs];
-    int nseg;
-};
-
 constexpr int kAttnMaxHeads = 256;
 constexpr int kAttnFusedMaxSeq = 256;  // up to this launch size attention runs as one workgroup per head
 constexpr int kAttnMaxChunks = 4;      // ranges of positions whose partial P.V sums the O projection adds up
@@ -203,53 +165,6 @@ __device__ __forceinline__ float lane_xor_sum(float v) {
     float a = v, b = v;
     if (OFF == 16) swap16(a, b); else swap32(a, b);
     return a + b;
-}
-
-// Touch the 128-byte lines of a prefetch plan that belong to XCD `xcd`, as workgroup `rank` of the `nranks` workgroups
-// (of T threads) that share the job on that XCD: one dword per line.  The lines of all segments form one index space
-// that the threads deal out among themselves, U to a thread per round, so that a round is one trip to memory whatever
-// the mix of large and small segments.  The loads are ordinary loads whose values are folded into a word that an empty
-// asm statement consumes at the end, so the compiler keeps them and does their wait-count bookkeeping itself.  (A load
-// issued from inside an asm statement returns into its register long after the compiler has given that register to
-// something else.)
-template <int T>
-__device__ __forceinline__ void prefetch_lines(const awq_prefetch_plan& plan, int xcd, int rank, int nranks) {
-    constexpr int U = 2;
-    auto lines_here = [&](const awq_prefetch_seg& sg) -> uint32_t {  // lines of this segment that belong to this XCD
-        const uint32_t my_blocks = sg.nblocks ? (sg.nblocks + 7 - (uint32_t)xcd) >> 3 : 1u;
-        return my_blocks * sg.lines_per_block;
-    };
-    uint32_t total = 0;
-    for (int s = 0; s < plan.nseg; s++) total += lines_here(plan.seg[s]);
-    if (total == 0) return;
-    const uint32_t stride = (uint32_t)nranks * T, first = (uint32_t)rank * T + threadIdx.x;
-    uint32_t seen = 0;
-    for (uint32_t i0 = first; i0 < total; i0 += U * stride) {  // (threads past the end skip the round: nothing else needs them)
-        uint32_t v[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            uint32_t i = i0 + u * stride;
-            if (i >= total) i = total - 1;  // a line somebody else touches too
-            int s = 0;
-            uint32_t n = lines_here(plan.seg[0]);
-            while (i >= n) {  // (total > i, so this ends inside the plan)
-                i -= n;
-                n = lines_here(plan.seg[++s]);
-            }
-            const awq_prefetch_seg sg = plan.seg[s];
-            const uintptr_t base = reinterpret_cast<uintptr_t>(sg.base);
-            const uint32_t blk = __umulhi(i, sg.inv_lines), line = i - blk * sg.lines_per_block;
-            const uintptr_t span = sg.nblocks ? (uintptr_t)sg.block_bytes * sg.nblocks : (uintptr_t)sg.block_bytes;
-            const uintptr_t start = sg.nblocks ? base + (uintptr_t)sg.block_bytes * ((uint32_t)xcd + 8 * blk) : base;
-            uintptr_t a = (start & ~(uintptr_t)127) + (uintptr_t)line * 128;
-            if (a < base) a = base;
-            if (a > base + span - 4) a = base + span - 4;  // alignment slack past the end: clamped onto the last dword
-            v[u] = *reinterpret_cast<const uint32_t*>(a);
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) seen ^= v[u];
-    }
-    asm volatile("" ::"v"(seen));
 }
 
 // Sum within each aligned group of 16 lanes (a DPP row); every lane of the

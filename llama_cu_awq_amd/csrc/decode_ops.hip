@@ -368,20 +368,12 @@ __global__ __launch_bounds__(1024) void attn_pv_partial_kernel(float* part, cons
 // hundred KB per head, so the launch count matters more than the parallelism); NS workgroups per head each take a
 // slice of the value dimensions and compute the scores redundantly.  Same arithmetic and
 // rounding points as the two-pass kernels above; the fp16 scores are also left in att.
-// Workgroups with blockIdx.y >= NS have no head: they pull what `pf` lists into the L2 of the XCD they run on, for the
-// launches that follow (this kernel moves a few hundred KB; HBM is otherwise idle while it runs).
 template <int LP, int NS>
 __global__ __launch_bounds__(1024) void attn_fused_kernel(uint16_t* output, uint16_t* att, const uint16_t* q,
                                                           const uint16_t* key_cache, const uint16_t* value_cache, int num_heads,
                                                           int head_size, int kv_mul, int row_stride, float alpha,
-                                                          const int* pPos, int max_seq_len, const awq_prefetch_plan pf) {
+                                                          const int* pPos, int max_seq_len) {
     extern __shared__ float fsm[];
-    if (blockIdx.y >= NS) {
-        // gridDim.x is a multiple of 8 and workgroups are dealt to the XCDs in turn, x fastest
-        const int per_xcd = gridDim.x >> 3;
-        prefetch_lines<1024>(pf, blockIdx.x & 7, (blockIdx.y - NS) * per_xcd + (blockIdx.x >> 3), (gridDim.y - NS) * per_xcd);
-        return;
-    }
     // LDS was sized for max_seq_len positions by the launcher; a position beyond it (a caller that sized the launch
     // from a stale position) must not run past that
     const int size = min(*pPos + 1, max_seq_len);
@@ -570,24 +562,14 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* x, int siz
 template <int LP>
 int launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const uint16_t* key_cache,
                      const uint16_t* value_cache, uint16_t* att, int num_heads, int head_size, int kv_mul, int max_seq_len,
-                     const int* pos, const awq_prefetch_plan* prefetch) {
+                     const int* pos) {
     const int row_stride = num_heads * head_size / kv_mul;
     const float alpha = (float)(1.0 / sqrt((double)head_size));
     if (max_seq_len <= kAttnFusedMaxSeq) {
         const size_t lds = (size_t)attention_head_lds_floats(max_seq_len, head_size, 16) * sizeof(float);
         // two workgroups per head (halves of the value dimensions): +0.4 .. 0.7 % tokens/s at 7B; four: no better
-        const int gx = (num_heads + 7) & ~7;
-        awq_prefetch_plan plan;
-        plan.nseg = 0;
-        int extra = 0;
-        if (prefetch && prefetch->nseg > 0) {
-            // the compute units the heads leave idle, one prefetching workgroup each
-            plan = *prefetch;
-            extra = (ctx->cus - 2 * gx) / gx;
-            if (extra < 1) extra = 1;
-        }
-        awq_launch(ctx, attn_fused_kernel<LP, 2>, dim3(gx, 2 + extra), dim3(1024), lds, output, att, q,
-                           key_cache, value_cache, num_heads, head_size, kv_mul, row_stride, alpha, pos, max_seq_len, plan);
+        awq_launch(ctx, attn_fused_kernel<LP, 2>, dim3((num_heads + 7) & ~7, 2), dim3(1024), lds, output, att, q,
+                           key_cache, value_cache, num_heads, head_size, kv_mul, row_stride, alpha, pos, max_seq_len);
         return awq_check_launch("attn_fused");
     }
     awq_launch(ctx, attn_scores_kernel<LP>, dim3(div_up(max_seq_len, 64), num_heads), dim3(256), 0, att, q,
@@ -638,29 +620,6 @@ int awq_launch_attention_partial(awq_ctx* ctx, float* part, int* chunks_out, con
     return awq_check_launch("attn_pv_partial");
 }
 
-// Internal: awq_attention with an optional list of memory that the launch's idle workgroups pull into L2 for the
-// launches behind it (used by the one-launch form only; the longer forms keep HBM busy themselves).
-int awq_launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const uint16_t* key_cache, const uint16_t* value_cache,
-                         uint16_t* att, int num_heads, int head_size, int kv_mul, int max_seq_len, const int* pos,
-                         const awq_prefetch_plan* prefetch) {
-    if (int r = awq_bind(ctx)) return r;
-    AWQ_REQUIRE(output && q && key_cache && value_cache && att && pos, AWQ_ERR_ARG, "null pointer");
-    AWQ_REQUIRE(num_heads > 0 && num_heads <= kAttnMaxHeads, AWQ_ERR_SHAPE, "num_heads out of range");
-    AWQ_REQUIRE(kv_mul > 0 && num_heads % kv_mul == 0, AWQ_ERR_SHAPE, "kv_mul must divide num_heads");
-    AWQ_REQUIRE(max_seq_len > 0, AWQ_ERR_SHAPE, "max_seq_len must be positive");
-    switch (head_size) {
-        case 64:
-            return launch_attention<8>(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos, prefetch);
-        case 128:
-            return launch_attention<16>(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos, prefetch);
-        case 256:
-            return launch_attention<32>(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos, prefetch);
-        default:
-            awq_set_error("awq_attention: head_size %d unsupported (64, 128 or 256)", head_size);
-            return AWQ_ERR_SHAPE;
-    }
-}
-
 // Internal: fp16 matvec with optional fused RMSNorm of x (norm_out must not alias x).
 int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
                           const uint16_t* norm_w, uint16_t* norm_out) {
@@ -706,7 +665,22 @@ int awq_rope(awq_ctx* ctx, uint16_t* q, uint16_t* k, int num_heads, int num_kv_h
 
 int awq_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const uint16_t* key_cache, const uint16_t* value_cache,
                   uint16_t* att, int num_heads, int head_size, int kv_mul, int max_seq_len, const int* pos) {
-    return awq_launch_attention(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos, nullptr);
+    if (int r = awq_bind(ctx)) return r;
+    AWQ_REQUIRE(output && q && key_cache && value_cache && att && pos, AWQ_ERR_ARG, "null pointer");
+    AWQ_REQUIRE(num_heads > 0 && num_heads <= kAttnMaxHeads, AWQ_ERR_SHAPE, "num_heads out of range");
+    AWQ_REQUIRE(kv_mul > 0 && num_heads % kv_mul == 0, AWQ_ERR_SHAPE, "kv_mul must divide num_heads");
+    AWQ_REQUIRE(max_seq_len > 0, AWQ_ERR_SHAPE, "max_seq_len must be positive");
+    switch (head_size) {
+        case 64:
+            return launch_attention<8>(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos);
+        case 128:
+            return launch_attention<16>(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos);
+        case 256:
+            return launch_attention<32>(ctx, output, q, key_cache, value_cache, att, num_heads, head_size, kv_mul, max_seq_len, pos);
+        default:
+            awq_set_error("awq_attention: head_size %d unsupported (64, 128 or 256)", head_size);
+            return AWQ_ERR_SHAPE;
+    }
 }
 
 int awq_attention_partial(awq_ctx* ctx, float* part, int* chunks, const uint16_t* q, const uint16_t* key_cache,

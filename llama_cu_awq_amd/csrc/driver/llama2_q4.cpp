@@ -4,7 +4,7 @@
 //   llama2_q4 <checkpoint> [-n steps] [-i prompt] [-f prompt_file] [-t temperature] [-p top_p] [-s seed]
 //             [-z tokenizer] [-y system_prompt] [-x none] [-q dataset]
 // Extra (not in the reference): -g 0|1 graph replay (default 1), -e 0|1 ignore EOS (default 0),
-//   -m reference|fused|persistent schedule (default fused), -b 0|1 batched prompt prefill (default 0).
+//   -m reference|fused|persistent schedule (default fused; persistent is experimental and about 2.3x slower), -b 0|1 batched prompt prefill (default 0).
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -40,7 +40,7 @@ static void error_usage(char* argv[]) {
     fprintf(stderr, "  -y <string> (optional) system prompt (accepted, unused, as in the reference)\n");
     fprintf(stderr, "  -q <string> dataset file (accepted, ignored: no perplexity mode)\n");
     fprintf(stderr, "  -g <0|1>    replay recorded launch sequences (hipGraph), default 1\n");
-    fprintf(stderr, "  -m <string> schedule: reference|fused|persistent, default fused\n");
+    fprintf(stderr, "  -m <string> schedule: reference|fused|persistent (experimental, ~2.3x slower), default fused\n");
     fprintf(stderr, "  -b <0|1>    consume the prompt in one batched prefill pass, default 0\n");
     fprintf(stderr, "  -e <0|1>    keep generating past the end-of-sequence token, default 0\n");
     fprintf(stderr, "  -d <0|1>    print the GPU time of every token, default 0\n");

@@ -1,7 +1,8 @@
 // Byte-fallback BPE tokenizer over a llama2.c-format tokenizer.bin (the file the reference ships and its
 // tokenizer.h reads: uint32 max_token_length, then per token {float score, int32 len, bytes}).
 // Same observable behaviour as the reference's build_tokenizer / encode / decode / safe_printf
-// (tokenizer.h:35-223); the implementation is this project's own (hash map lookup instead of qsort+bsearch).
+// (tokenizer.h:35-223); the implementation is this project's own (a vector of (string, id) pairs sorted once with
+// std::stable_sort and searched by bisection, where the reference calls qsort and bsearch).
 #pragma once
 
 #include <ctype.h>

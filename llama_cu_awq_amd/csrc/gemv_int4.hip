@@ -47,18 +47,34 @@ struct GemvParams {
     int head_size;           // for the fused RoPE row pairing
     const float* xpart;      // PARTS form: x is the sum of `xparts` fp32 vectors K floats apart, rounded to fp16
     int xparts;
+    // Filled in by launch().  Everything a wave needs before it can request its first packed weights is a handful of
+    // scalar instructions on these: the compute unit's one scalar unit serves all of its waves, and with 16 to 24 waves
+    // arriving at once every scalar instruction of the prologue costs all of them a cycle (a division by the grid size
+    // and 64-bit row offsets had put the first weight request 0.8 us, in the QKV kernel 1.6 us, behind the wave's start).
+    int gx;                  // workgroups along x (= gridDim.x, without the trip to the dispatch packet)
+    int groups_q, groups_rem;  // row groups per workgroup: groups_q, and one more for workgroups below groups_rem
+    int half_shift;          // log2(head_size / 2) for the fused RoPE pairing (head sizes are powers of two there)
+    uint32_t wbytes, zbytes, sbytes;  // bytes per row of weights, zeros, scales (32-bit offsets: a matrix is below 4 GiB)
+#ifdef AWQ_STAMPS
+    long long* stamps;       // instrumented build: 6 wall-clock stamps (10 ns ticks) per workgroup, or null
+#endif
 };
+
+#ifdef AWQ_STAMPS
+#define AWQ_STAMP(i) do { if (p.stamps && threadIdx.x == 0) stamp_[i] = wall_clock64(); } while (0)
+#else
+#define AWQ_STAMP(i) do { } while (0)
+#endif
 
 enum { KIND_SINGLE = 0, KIND_QKV = 1, KIND_FFN = 2 };
 
 // Logical index li of a workgroup's row space -> matrix row.  With ROPE, consecutive indices (2j, 2j+1) are the two
 // rows (i, i + head/2) of one rotation pair, so that one wave holds both.
 template <bool ROPE>
-__device__ __forceinline__ int map_row(int li, int head_size) {
+__device__ __forceinline__ int map_row(int li, int half_shift) {
     if (!ROPE) return li;
-    const int half = head_size >> 1;
     const int pi = li >> 1;
-    return (pi / half) * head_size + (pi % half) + (li & 1) * half;
+    return ((pi >> half_shift) << (half_shift + 1)) + (pi & ((1 << half_shift) - 1)) + ((li & 1) << half_shift);
 }
 
 // SPLIT (1, 2 or 4): a row takes 64 / SPLIT lanes, and the SPLIT parts of a wave work on SPLIT rows side by side (QKV
@@ -72,17 +88,20 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     static_assert(!PARTS || (!NORM && KIND == KIND_SINGLE), "partial-sum input only for the plain single-matrix form");
     extern __shared__ u32x4 xs[];
     __shared__ float red[W + 1];
+#ifdef AWQ_STAMPS
+    long long stamp_[6] = {0, 0, 0, 0, 0, 0};
+#endif
+    AWQ_STAMP(0);  // entry
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: row addresses stay scalar
     const int C = p.C;
-    const int pwh = C * 4;
     static_assert(SPLIT == 1 || SPLIT == 2 || SPLIT == 4, "a row takes 64, 32 or 16 lanes");
     constexpr bool HALF = SPLIT > 1;        // (the name from when two was the only split)
     constexpr int LPR = 64 / SPLIT;        // lanes per row
     constexpr int RW = SPLIT * R;          // rows (FFN: gate/up pairs) of a wave per row group
     const int hf = HALF ? lane / LPR : 0;  // which of the wave's SPLIT rows this lane works on
     const int ll = HALF ? lane % LPR : lane;
-    const int P = (C + LPR - 1) / LPR;  // passes per row (per SPLIT rows)
+    const int P = (int)(((uint32_t)C + LPR - 1) / LPR);  // passes per row (per SPLIT rows)
     float* ca = reinterpret_cast<float*>(xs + 4 * C);
     const int which = (KIND == KIND_QKV) ? blockIdx.y : 0;
     const bool rope_here = ROPE && which != 2;
@@ -101,21 +120,21 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
         out_base += (size_t)loff + (size_t)(*p.pos) * p.N;
         loff = -1;
     }
-    // (unconditional: a load inside a branch is waited for before the next one is issued; without a position the word
-    // read is the head of the packed weights, the one pointer every form of the kernel has, and goes unused)
-    int zero = 0;
-    asm volatile("" : "+v"(zero));
-    const int* pos_word = p.pos ? p.pos : reinterpret_cast<const int*>(m0.w);
-    const int pos_now = pos_word[zero];
+    // (it is the first load of the wave, so whether the branch is taken changes nothing for the loads counted behind it)
+    int pos_now = 0;
+    if (KIND != KIND_FFN && p.pos) {
+        int zero = 0;
+        asm volatile("" : "+v"(zero));
+        pos_now = p.pos[zero];
+    }
 
     // This workgroup's row groups (W waves x R rows each).  A wave walks its rows as a sequence of stages (group-major,
     // then pass); D stages are in flight at any time.  The sequence is padded to a multiple of D with repeats of the
     // last stage, which are loaded (same addresses again) but not accumulated, so that the number of loads between a
     // stage's request and its use is a compile-time constant.
     // The workgroup takes row groups blockIdx.x, blockIdx.x + gridDim.x, ... (x is staged once for all of them).
-    const int groups_total = (p.N + W * RW - 1) / (W * RW);
-    const int g_begin = blockIdx.x, g_stride = gridDim.x;
-    const int total = ((groups_total - 1 - g_begin) / g_stride + 1) * P;
+    const int g_begin = blockIdx.x, g_stride = p.gx;
+    const int total = (p.groups_q + ((int)blockIdx.x < p.groups_rem ? 1 : 0)) * P;
 
     // ---- load cursor
     const uint32_t* wrow[NS];
@@ -130,27 +149,30 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int li = min((g * W + wave) * RW + SPLIT * r, p.N - 1);  // indices past N are recomputed, never stored
-            const int row = rope_here ? map_row<true>(li, p.head_size) : li;
+            const int row = rope_here ? map_row<true>(li, p.half_shift) : li;
             if (HALF) {
                 const int li_own = min((g * W + wave) * RW + SPLIT * r + hf, p.N - 1);
-                const int drow = (rope_here ? map_row<true>(li_own, p.head_size) : li_own) - row;
-                hoff_w[r] = (uint32_t)(drow * pwh * 4);
-                hoff_z[r] = (uint32_t)(drow * p.pzh * 4);
-                hoff_s[r] = (uint32_t)(drow * p.sh * 2);
+                const int drow = (rope_here ? map_row<true>(li_own, p.half_shift) : li_own) - row;
+                hoff_w[r] = (uint32_t)drow * p.wbytes;
+                hoff_z[r] = (uint32_t)drow * p.zbytes;
+                hoff_s[r] = (uint32_t)drow * p.sbytes;
                 hoff_r[r] = (uint32_t)(drow * 2);
             }
-            resrow[r] = out_base + row;  // (the residual form never writes KV-cache rows: no position offset)
+            resrow[r] = reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(out_base) + (uint32_t)row * 2u);  // (the residual form never writes KV-cache rows: no position offset)
+            // (byte offsets formed in 32 bits: one scalar multiply and one 64-bit add per pointer)
+            const uint32_t ow = (uint32_t)row * p.wbytes, oz = (uint32_t)row * p.zbytes, os = (uint32_t)row * p.sbytes;
+            auto at = [](const auto* base, uint32_t off) { return reinterpret_cast<decltype(base)>(reinterpret_cast<const char*>(base) + off); };
             if (KIND == KIND_FFN) {
-                wrow[2 * r] = m0.w + (size_t)row * pwh;
-                zrow[2 * r] = m0.z + (size_t)row * p.pzh;
-                srow[2 * r] = m0.s + (size_t)row * p.sh;
-                wrow[2 * r + 1] = m1.w + (size_t)row * pwh;
-                zrow[2 * r + 1] = m1.z + (size_t)row * p.pzh;
-                srow[2 * r + 1] = m1.s + (size_t)row * p.sh;
+                wrow[2 * r] = at(m0.w, ow);
+                zrow[2 * r] = at(m0.z, oz);
+                srow[2 * r] = at(m0.s, os);
+                wrow[2 * r + 1] = at(m1.w, ow);
+                zrow[2 * r + 1] = at(m1.z, oz);
+                srow[2 * r + 1] = at(m1.s, os);
             } else {
-                wrow[r] = m0.w + (size_t)row * pwh;
-                zrow[r] = m0.z + (size_t)row * p.pzh;
-                srow[r] = m0.s + (size_t)row * p.sh;
+                wrow[r] = at(m0.w, ow);
+                zrow[r] = at(m0.z, oz);
+                srow[r] = at(m0.s, os);
             }
         }
     };
@@ -219,7 +241,7 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
                 for (int r = 0; r < (HALF ? R : R - 1); r += (HALF ? 1 : 2)) {
                     const int li = li0 + (HALF ? SPLIT * r + hf : r);
                     if (li < p.N) {
-                        const int row = map_row<true>(li, p.head_size);
+                        const int row = map_row<true>(li, p.half_shift);
                         const float v0 = half_bits_to_float(float_to_half_bits(sum[r]));
                         const float v1 = half_bits_to_float(float_to_half_bits(HALF ? second[r] : sum[HALF ? r : r + 1]));
                         const float2 c = cs_tab[row % half];
@@ -289,12 +311,20 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
         load_parts<W>(pr, xa);
     else
         load_x<W, NORM>(xr, xa);
+    AWQ_STAMP(1);  // x requested
     Stage<NS> st[D];
     set_rows(lg);
 #pragma unroll
-    for (int d = 0; d < D; d++) issue(st[d]);
+    for (int d = 0; d < D; d++) {
+        issue(st[d]);
+#ifdef AWQ_STAMPS
+        if (d == 0) AWQ_STAMP(2);  // first stage requested
+#endif
+    }
+    AWQ_STAMP(3);  // all D stages requested
     if constexpr (PARTS) combine_x<W>(xr, pr, xa);
     stage_x<W, NORM>(xs, ca, xa, red, xr);
+    AWQ_STAMP(4);  // x staged
     const int rounds = (total + D - 1) / D;
     for (int r = 1; r < rounds; r++) {
 #pragma unroll
@@ -305,7 +335,13 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     }
 #pragma unroll
     for (int d = 0; d < D; d++) consume(st[d]);
-
+#ifdef AWQ_STAMPS
+    if (p.stamps && threadIdx.x == 0) {
+        stamp_[5] = wall_clock64();  // results stored
+        long long* o = p.stamps + 6 * (size_t)(blockIdx.y * gridDim.x + blockIdx.x);
+        for (int i = 0; i < 6; i++) o[i] = stamp_[i];
+    }
+#endif
 }
 
 // out[n*K + k] = half_rne((q - z) * s): exact fp32 product, one rounding.
@@ -334,6 +370,10 @@ int check_shape(int K, int N) {
     // llama2_q4.cu:368: "Unsupported matmul size"
     if (K <= 0 || N <= 0 || (K & 7) || (N & 7)) {
         awq_set_error("unsupported matmul size K=%d N=%d (both must be positive multiples of 8)", K, N);
+        return AWQ_ERR_SHAPE;
+    }
+    if ((size_t)N * (size_t)div_up(K, 32) * 16 >= ((size_t)1 << 32)) {
+        awq_set_error("matrix of K=%d N=%d exceeds the 4 GiB that 32-bit row offsets address", K, N);
         return AWQ_ERR_SHAPE;
     }
     if (K > kMaxStagedK) {
@@ -373,9 +413,11 @@ struct GemvPlan {
     int depth;   // stages in flight per wave (2, 3, 4)
 };
 
-// When set (by awq_gemv_geometry, on the calling thread), launch() reports the geometry it would launch with instead
-// of launching.
-thread_local awq_gemv_geometry_t* g_geometry_query = nullptr;
+#ifdef AWQ_STAMPS
+long long* g_stamps_base = nullptr;
+int g_stamps_stride = 0, g_stamps_launches = 0, g_stamps_next = 0;
+int g_stamps_grid[4096], g_stamps_bytes[4096];
+#endif
 
 template <int W, int R, int D, int KIND, bool ROPE, int SPLIT = 1>
 int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
@@ -388,13 +430,29 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
         const int cus = ctx->cus;
         if (gx > 3 * cus) gx = 3 * cus;
     }
-    if (g_geometry_query) {
-        g_geometry_query->rows_per_group = W * R * SPLIT;
-        g_geometry_query->groups = groups_total;
-        g_geometry_query->grid_x = gx;
-        g_geometry_query->paired_rows = ROPE ? 1 : 0;
-        return AWQ_OK;
+    p.gx = gx;
+    p.groups_q = groups_total / gx;
+    p.groups_rem = groups_total % gx;
+    p.half_shift = 0;
+    if (ROPE) {
+        while ((2 << p.half_shift) < p.head_size) p.half_shift++;
+        if ((2 << p.half_shift) != p.head_size) {
+            awq_set_error("%s: the fused rotation needs a power-of-two head size (got %d)", what, p.head_size);
+            return AWQ_ERR_SHAPE;
+        }
     }
+    p.wbytes = (uint32_t)p.C * 16u;
+    p.zbytes = (uint32_t)p.pzh * 4u;
+    p.sbytes = (uint32_t)p.sh * 2u;
+#ifdef AWQ_STAMPS
+    p.stamps = nullptr;
+    if (g_stamps_base && g_stamps_next < g_stamps_launches && (int)(gx * grid_y) <= g_stamps_stride) {
+        p.stamps = g_stamps_base + (size_t)g_stamps_next * g_stamps_stride * 6;
+        g_stamps_grid[g_stamps_next] = gx * grid_y;
+        g_stamps_bytes[g_stamps_next] = KIND * 1000 + W;
+        g_stamps_next++;
+    }
+#endif
     const dim3 grid(gx, grid_y);
     const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
     if constexpr (KIND == KIND_SINGLE && !ROPE && R == 1 && (W == 8 || W == 10 || W == 13)) {  // (partial-sum input comes with K <= 8192)
@@ -591,27 +649,19 @@ int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qwe
     return dispatch<KIND_FFN, false>(ctx, p, 1, "ffn_matvec_silu", plan_for(K, 1));
 }
 
-// Internal: the launch geometry the dispatcher picks for a product (nothing is launched).  kind: 0 single matrix
-// (norm: RMSNorm fused; parts: input as partial sums), 2 gate/up.  Row group g (rows_per_group consecutive rows, of both
-// matrices in the gate/up form) is read by workgroup g % grid_x.
-int awq_gemv_geometry(awq_ctx* ctx, int kind, int K, int N, int norm, int parts, awq_gemv_geometry_t* out) {
-    static const uint16_t dummy = 0;
-    GemvParams p;
-    fill_common(p, &dummy, K, N);
-    if (norm) p.norm_w = &dummy;
-    if (parts) {
-        p.xpart = reinterpret_cast<const float*>(&dummy);
-        p.xparts = parts;
-    }
-    g_geometry_query = out;
-    int r;
-    if (kind == 2)
-        r = dispatch<KIND_FFN, false>(ctx, p, 1, "geometry", plan_for(K, 1));
-    else
-        r = dispatch<KIND_SINGLE, false>(ctx, p, 1, "geometry", plan_for(K, 1));
-    g_geometry_query = nullptr;
-    return r;
+#ifdef AWQ_STAMPS
+// Instrumented build only: every int4 matrix-vector launch from now on writes its workgroups' stamps to
+// buf[launch][wg_stride][6]; returns how many launches have been recorded so far and their grid sizes / kinds.
+extern "C" int awq_debug_stamps(long long* buf, int wg_stride, int max_launches, int* grids_out, int* kinds_out) {
+    const int n = g_stamps_next;
+    if (grids_out) for (int i = 0; i < n; i++) { grids_out[i] = g_stamps_grid[i]; kinds_out[i] = g_stamps_bytes[i]; }
+    g_stamps_base = buf;
+    g_stamps_stride = wg_stride;
+    g_stamps_launches = max_launches > 4096 ? 4096 : max_launches;
+    g_stamps_next = 0;
+    return n;
 }
+#endif
 
 extern "C" {
 

@@ -28,10 +28,6 @@ int awq_launch_attention_partial(awq_ctx* ctx, float* part, int* chunks_out, con
                                  int max_seq_len, const int* pos);
 int awq_launch_matvec_int4_parts(awq_ctx* ctx, uint16_t* out, const float* part, int parts, const awq_qweight* w, int K, int N,
                                  int accum);
-int awq_launch_attention(awq_ctx* ctx, uint16_t* output, const uint16_t* q, const uint16_t* key_cache, const uint16_t* value_cache,
-                         uint16_t* att, int num_heads, int head_size, int kv_mul, int max_seq_len, const int* pos,
-                         const awq_prefetch_plan* prefetch);
-int awq_gemv_geometry(awq_ctx* ctx, int kind, int K, int N, int norm, int parts, awq_gemv_geometry_t* out);
 int awq_launch_argmax(awq_ctx* ctx, const uint16_t* logits, int size, int* tokens, volatile int* pos_host, int* pos_dev,
                       int write_token, int* tokens_mirror);
 // sampler.hip
@@ -110,10 +106,6 @@ struct awq_transformer {
     int* tokens_dev;  // device mirror of SharedData.tokens (the persistent kernel reads its input token here)
     float2* rope_table;  // [seq_len][head_size/2] (cos, sin)
     float* attn_part;    // [kAttnMaxChunks][dim] fp32 partial attention outputs of the position-split form
-    // per layer: what the idle workgroups of the one-launch attention pull into L2 for the O projection and the head of
-    // the gate/up product behind it (fused schedule)
-    std::vector<awq_prefetch_plan> attn_prefetch;
-    bool prefetch_on;
     // plan of the persistent per-token kernel
     bool tk_ok;
     char tk_why[160];  // why the persistent kernel cannot run this model, when !tk_ok
@@ -228,58 +220,6 @@ int alloc_state(awq_transformer* t) {
     return AWQ_OK;
 }
 
-// One int4 matrix as prefetch segments (weights, zeros, scales), `nblocks` row groups of `rows` rows from the top.
-void add_matrix_segments(awq_prefetch_plan& plan, const awq_qweight& w, int K, int rows, int nblocks) {
-    if (nblocks <= 0 || plan.nseg + 3 > kPrefetchSegs) return;
-    plan.seg[plan.nseg++] = awq_make_prefetch_seg(w.weight, (size_t)rows * packed_weight_height(K) * 4, (uint32_t)nblocks);
-    plan.seg[plan.nseg++] = awq_make_prefetch_seg(w.zeros, (size_t)rows * packed_zeros_height(K) * 4, (uint32_t)nblocks);
-    plan.seg[plan.nseg++] = awq_make_prefetch_seg(w.scales, (size_t)rows * scales_height(K) * 2, (uint32_t)nblocks);
-}
-
-void add_vector_segment(awq_prefetch_plan& plan, const void* p, size_t bytes) {
-    if (plan.nseg + 1 > kPrefetchSegs) return;
-    plan.seg[plan.nseg++] = awq_make_prefetch_seg(p, bytes, 0u);  // every XCD
-}
-
-// Per layer, what the one-launch attention's idle workgroups fetch: all of the O projection (it runs next and reads
-// nothing else of size) and as much of the first round of the gate/up product as the budget leaves, each line into
-// the L2 of the XCD whose workgroup will read it (row group g -> workgroup g % grid_x -> XCD g % 8, which holds when
-// grid_x is a multiple of 8 or every group has a workgroup of its own).
-int build_prefetch_plans(awq_transformer* t) {
-    const awq_config& c = t->cfg;
-    const char* env = getenv("AWQ_PREFETCH");
-    t->prefetch_on = env && env[0] == '1';  // (off unless asked for while it is being measured)
-    t->attn_prefetch.assign(c.n_layers, awq_prefetch_plan{});
-    awq_gemv_geometry_t go, gf;
-    if (int r = awq_gemv_geometry(t->ctx, 0, c.dim, c.dim, 0, 0, &go)) return r;
-    if (int r = awq_gemv_geometry(t->ctx, 2, c.dim, c.hidden_dim, 1, 0, &gf)) return r;
-    auto mapped = [](const awq_gemv_geometry_t& g) { return !g.paired_rows && (g.grid_x == g.groups || (g.grid_x & 7) == 0); };
-    const size_t row_bytes = (size_t)packed_weight_height(c.dim) * 4 + (size_t)packed_zeros_height(c.dim) * 4 + (size_t)scales_height(c.dim) * 2;
-    for (int l = 0; l < c.n_layers; l++) {
-        awq_prefetch_plan& plan = t->attn_prefetch[l];
-        plan.nseg = 0;
-        const awq_layer_weights& L = t->layers[l];
-        size_t used = 0;
-        if (mapped(go)) {
-            const int nblocks = c.dim / go.rows_per_group;  // whole groups only
-            add_matrix_segments(plan, L.wq_o, c.dim, go.rows_per_group, nblocks);
-            add_vector_segment(plan, t->s.x, (size_t)c.dim * 2);  // the residual the projection adds to
-            used = (size_t)nblocks * go.rows_per_group * row_bytes;
-        }
-        if (mapped(gf) && used < kPrefetchBudgetBytes) {
-            int nblocks = gf.groups < gf.grid_x ? gf.groups : gf.grid_x;  // the first row group of every workgroup
-            if (nblocks > c.hidden_dim / gf.rows_per_group) nblocks = c.hidden_dim / gf.rows_per_group;
-            const size_t block = 2 * (size_t)gf.rows_per_group * row_bytes;  // gate and up
-            const size_t fit = (kPrefetchBudgetBytes - used) / block;
-            if ((size_t)nblocks > fit) nblocks = (int)(fit & ~(size_t)7);
-            add_matrix_segments(plan, L.wq_gate, c.dim, gf.rows_per_group, nblocks);
-            add_matrix_segments(plan, L.wq_up, c.dim, gf.rows_per_group, nblocks);
-            if (nblocks > 0) add_vector_segment(plan, L.rms_ffn_weight, (size_t)c.dim * 2);
-        }
-    }
-    return AWQ_OK;
-}
-
 void release(awq_transformer* t) {
     if (!t) return;
     for (int m = 0; m < 2; m++)
@@ -329,7 +269,6 @@ awq_transformer* new_transformer(awq_ctx* ctx) {
     t->pf_rows = 0;
     t->pf_x = t->pf_xb = t->pf_q = t->pf_att = t->pf_hb = nullptr;
     t->issued_pos = 0;
-    t->prefetch_on = false;
     memset(&t->s, 0, sizeof(t->s));
     memset(t->captured, 0, sizeof(t->captured));
     return t;
@@ -599,8 +538,8 @@ int network_fused(awq_transformer* t, int seq_len_bin) {
                 r = awq_launch_attention_partial(ctx, t->attn_part, &parts, s.q, s.key_cache + loff, s.value_cache + loff, s.att,
                                                  p.n_heads, head_size, kv_mul, seq_len_bin, pPos);
             else
-                r = awq_launch_attention(ctx, s.xb, s.q, s.key_cache + loff, s.value_cache + loff, s.att, p.n_heads, head_size,
-                                         kv_mul, seq_len_bin, pPos, t->prefetch_on ? &t->attn_prefetch[l] : nullptr);
+                r = awq_attention(ctx, s.xb, s.q, s.key_cache + loff, s.value_cache + loff, s.att, p.n_heads, head_size, kv_mul,
+                                  seq_len_bin, pPos);
             if (r) return r;
         }
         {
@@ -701,7 +640,6 @@ int awq_transformer_load_image(awq_ctx* ctx, const void* image, size_t bytes, aw
     }
     map_tensors(t);
     r = alloc_state(t);
-    if (r == AWQ_OK) r = build_prefetch_plans(t);
     if (r == AWQ_OK) r = plan_token_kernel(t);
     if (r) {
         release(t);
@@ -789,7 +727,6 @@ int awq_transformer_load_file(awq_ctx* ctx, const char* checkpoint_path, awq_tra
     }
     map_tensors(t);
     r = alloc_state(t);
-    if (r == AWQ_OK) r = build_prefetch_plans(t);
     if (r == AWQ_OK) r = plan_token_kernel(t);
     if (r) {
         release(t);

@@ -100,3 +100,22 @@ def test_cli_argument_validation(model_file):
     assert r.returncode == 0 and b"achieved tok/s" in r.stdout
     r2 = subprocess.run([CLI, path, "-n", "12", "-t", "0.8", "-p", "0.9", "-s", "7", "-i", "Hi", "-z", TOKBIN, "-e", "1"], capture_output=True, timeout=120)
     assert r.stdout.split(b"achieved")[0] == r2.stdout.split(b"achieved")[0]  # same seed, same text
+
+
+def test_cli_per_token_timings(model_file):
+    """-d 1, the reference's DUMP_PER_TOKEN_TIMINGS switch (llama2_q4.cu:592-600): every pass through the network prints
+    ` t: <milliseconds> ` (the event pair around network + sampler), one per pass, and the text between them is the run's
+    usual output."""
+    path, img = model_file
+    prompt, steps = "Write a poem on GPUs", 20
+    base = subprocess.run([CLI, path, "-n", str(steps), "-t", "0", "-i", prompt, "-z", TOKBIN, "-e", "1"], capture_output=True, timeout=120)
+    timed = subprocess.run([CLI, path, "-n", str(steps), "-t", "0", "-i", prompt, "-z", TOKBIN, "-e", "1", "-d", "1"], capture_output=True, timeout=120)
+    assert base.returncode == 0 and timed.returncode == 0, timed.stderr.decode()
+    body = timed.stdout.split(b"Encoding Prompt... Done!\n", 1)[1].split(b"\n\n[GPU: 0] achieved tok/s:", 1)[0]
+    stamps = re.findall(rb" t: ([0-9.eE+-]+) ", body)
+    assert len(stamps) == steps  # one pass per loop iteration, positions 0 .. steps-1 (llama2_q4.cu:716)
+    assert all(0.0 < float(x) < 1000.0 for x in stamps)
+    # with the stamps taken out, the text is that of the plain run
+    plain = base.stdout.split(b"Encoding Prompt... Done!\n", 1)[1].split(b"\n\n[GPU: 0] achieved tok/s:", 1)[0]
+    assert re.sub(rb" t: [0-9.eE+-]+ ", b"", body) == plain
+    assert b" t: " not in plain
