@@ -106,3 +106,63 @@ def test_prefill_in_two_parts_equals_one(ctx):
     a, b = states
     assert a[3] == b[3] == 70 and a[4] == b[4]
     assert rel_l2(f16(a[0]), f16(b[0])) <= 1e-3 and rel_l2(f16(a[1]), f16(b[1])) <= 1e-3 and rel_l2(f16(a[2]), f16(b[2])) <= 2e-3
+
+
+# 128-wide heads and a context past what the batched attention keeps in LDS (1920 positions): the tokens beyond that bound
+# go through the matrix-vector path one at a time inside the same call (position hand-over, token list, the
+# position-split attention from 1024 positions on).
+CFG_LONG2K = dict(dim=256, hidden_dim=512, n_layers=2, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=2176, rope_theta=10000.0)
+
+
+def test_prefill_past_the_batched_attention_bound(ctx):
+    cfg, n_prompt = CFG_LONG2K, 2000
+    img = synth.make_model_image(cfg, seed=33, scale_mult=0.5)
+    prompt = synth.prompt_tokens(33, n_prompt, cfg["vocab_size"])
+    o = oracle.Model(img)
+    o.reset(prompt)
+    for i in range(n_prompt):
+        o.forward(i >= n_prompt - 1)
+    kv_dim, L, seq, vocab = cfg["dim"], cfg["n_layers"], cfg["seq_len"], cfg["vocab_size"]
+    want_kv = {n: f16(o.buffer(n, L * seq * kv_dim)).reshape(L, seq, kv_dim)[:, :n_prompt].copy() for n in ("key_cache", "value_cache")}
+    want_logits = f16(o.buffer("logits", vocab)).copy()
+    want_next = o.tokens(n_prompt + 1)[n_prompt]
+
+    def state(t):
+        ctx.sync()
+        kv = {n: f16(t.download(n, L * seq * kv_dim)).reshape(L, seq, kv_dim)[:, :n_prompt] for n in ("key_cache", "value_cache")}
+        return kv, f16(t.download("logits", vocab)), t.token(n_prompt), t.pos
+
+    results = {}
+    for name, parts in (("one call", (2000,)), ("1900 + 100", (1900, 100)), ("token by token", None)):
+        t = A.Transformer(ctx, image=img)
+        t.reset(prompt)
+        if parts is None:
+            for i in range(n_prompt):
+                t.forward(i >= n_prompt - 1, False, A.SCHEDULE_FUSED)
+        else:
+            for i, n in enumerate(parts):
+                t.prefill(n, gen_token=(i == len(parts) - 1))
+        results[name] = state(t)
+        kv, logits, nxt, pos = results[name]
+        assert pos == n_prompt, name
+        for n in ("key_cache", "value_cache"):
+            for l in range(L):
+                assert rel_l2(kv[n][l], want_kv[n][l]) <= 1e-2, (name, n, l)
+                # the rows written one at a time past the bound, on their own
+                assert rel_l2(kv[n][l][1920:], want_kv[n][l][1920:]) <= 1e-2, (name, n, l)
+        assert rel_l2(logits, want_logits) <= 1e-2, name
+        assert nxt == want_next, name
+        # decoding continues from there
+        for i in range(4):
+            ctx.sync()
+            t.forward(True, False, A.SCHEDULE_FUSED)
+        ctx.sync()
+        assert t.pos == n_prompt + 4
+        results[name] += ([t.token(n_prompt + 1 + i) for i in range(4)],)
+        t.close()
+    for i in range(4):
+        o.forward(True)
+    want_more = o.tokens(n_prompt + 5)[n_prompt + 1 :]
+    for name, r in results.items():
+        assert r[4] == want_more, name
+    o.close()
