@@ -312,6 +312,10 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     else
         load_x<W, NORM>(xr, xa);
     AWQ_STAMP(1);  // x requested
+    // Norm-fused forms: every wave's share of x is requested before any wave of the workgroup requests weights.  The
+    // staging needs all shares, and a share requested behind another wave's weights waits in the compute unit's queue
+    // until those have been delivered (+0.7 % tokens/s at 7B; the plain forms, whose staging is short, lose by it).
+    if (NORM) __builtin_amdgcn_s_barrier();
     Stage<NS> st[D];
     set_rows(lg);
 #pragma unroll
