@@ -6,8 +6,8 @@ random prompt as warm-up and times exactly 256 decode steps; weights are random 
 real layout and distributions, resident in HBM before the timed region starts.
 
 Prints ONE JSON line: tokens/s (`value`) of the run the flags ask for; `config1`, the benchmark's own run (16-token
-prompt + 256 decode steps from position 0) whatever the flags were; `config2` and `config3`, short runs of the 13B shape
-from a KV cache pre-filled to position 1536 and of the 33B shape; the roofline of the dominant kernel as the timed
+prompt + 256 decode steps from position 0) whatever the flags were; `config2` and `config3`, 256 decode steps of the 13B
+shape from a KV cache pre-filled to position 1536 and of the 33B shape; the roofline of the dominant kernel as the timed
 schedule launches it (RMSNorm-fused gate/up int4 matrix-vector product, timed live with HIP events over the 32
 layers' distinct weights); `config0`, the single 4096 x 4096 product back to back on one stream and dealt over 2 and 4
 plain streams; the 512-token prefill; and the CPU oracle timed on a bounded sample of the same workload.
@@ -321,7 +321,7 @@ def main():
         model.close()
         model = None
         del image
-        for key, name, start, steps, scale in (("config2", "13b", 1536, 64, 1.0), ("config3", "33b", 0, 32, 0.5)):
+        for key, name, start, steps, scale in (("config2", "13b", 1536, 256, 1.0), ("config3", "33b", 0, 256, 0.5)):
             xcfg = {"13b": synth.CONFIG_13B, "33b": synth.CONFIG_33B}[name]
             t0 = time.time()
             ximg = synth.make_model_image(xcfg, seed=args.seed, threads=min(16, os.cpu_count() or 8), scale_mult=scale)
