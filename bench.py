@@ -312,6 +312,21 @@ def main():
             "sample": f"{args.cpu_tokens} tokens of the same {args.config} model (positions 1..{args.cpu_tokens}) through the scalar C++/OpenMP oracle, after 1 untimed token",
         }
         o.close()
+        # configuration 0 on the host: the single 4096 x 4096 product through the oracle, 32 distinct matrices (279 MB)
+        # x 4 rounds
+        mats = [synth.make_qweight(synth.stream_key(args.seed, "config0", i), 4096, 4096) for i in range(32)]
+        x0 = synth.normal_f16(synth.stream_key(args.seed, "config0", "x"), 4096)
+        y0 = np.zeros(4096, dtype=np.float16)
+        for w, z, sc in mats[:4]:
+            oracle.matvec_int4(y0, x0, w, z, sc, 4096, 4096)
+        c0 = time.perf_counter()
+        for _ in range(4):
+            for w, z, sc in mats:
+                oracle.matvec_int4(y0, x0, w, z, sc, 4096, 4096)
+        c_us = (time.perf_counter() - c0) * 1e6 / (4 * len(mats))
+        cpu["config0"] = {"us_per_product": round(c_us, 1), "gbps": round((qweight_bytes(4096, 4096) + 4 * 4096) / c_us / 1e3, 2),
+                          "sample": "128 products over 32 distinct 4096 x 4096 matrices"}
+        del mats
 
     # ---- configurations 2 and 3 (13B shape from a cache pre-filled to 1536; 33B shape), compact, after everything that
     # needs the 7B model.  The 33B image takes half the benchmark's scale range: with the full range the residual stream
