@@ -80,6 +80,7 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--config", default="7b", choices=["7b", "13b", "33b"])
+    ap.add_argument("--scale-mult", type=float, default=None, help="multiplies the weights' scale range U[0.002, 0.02]; default 1.0, and 0.5 for --config 33b (60 layers leave fp16 range at 1.0)")
     ap.add_argument("--start-pos", type=int, default=0, help="pre-fill the KV cache with N(0,1) up to this position first")
     ap.add_argument("--schedule", default="fused", choices=["persistent", "fused", "reference"])
     ap.add_argument("--no-graph", action="store_true")
@@ -106,7 +107,8 @@ def main():
     use_graph = not args.no_graph
 
     t0 = time.time()
-    image = synth.make_model_image(cfg, seed=args.seed, threads=min(16, os.cpu_count() or 8))
+    scale_mult = args.scale_mult if args.scale_mult is not None else (0.5 if args.config == "33b" else 1.0)
+    image = synth.make_model_image(cfg, seed=args.seed, threads=min(16, os.cpu_count() or 8), scale_mult=scale_mult)
     print(f"[bench] model image {image.nbytes / 1e9:.2f} GB generated in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
     ctx = A.Context(0)
     t0 = time.time()

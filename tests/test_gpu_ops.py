@@ -238,7 +238,7 @@ def test_zero_weights_leave_residual(ctx):
     assert np.abs(f16(dout.download(np.uint16)).astype(np.float64)).max() <= 1e-5
 
 
-@pytest.mark.parametrize("K,N", [(4096, 4096), (5120, 5120), (256, 64)])
+@pytest.mark.parametrize("K,N", [(4096, 4096), (5120, 5120), (256, 64), (6656, 6656), (512, 6656)])  # the last two: 10-wave workgroups, the last one partly filled
 def test_qkv_matvec(ctx, K, N):
     mats = [_case(K, N, t)[:3] for t in (10, 11, 12)]
     x = _case(K, N, 13)[3]
