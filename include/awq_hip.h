@@ -228,8 +228,9 @@ int awq_transformer_set_pos(awq_transformer* t, int pos, int token);
 #define AWQ_SCHEDULE_PERSISTENT 2
 int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, int mode);
 
-/* Record and instantiate ahead of time the launch sequences that awq_transformer_forward(use_graph != 0) replays for
- * positions below max_positions (one per sequence-length bin, llama2_q4.cu:553-575, where the reference records a bin
+/* Record and instantiate ahead of time the launch sequences that awq_transformer_forward and
+ * awq_transformer_forward_logits (use_graph != 0) replay for positions below max_positions (per sequence-length bin,
+ * llama2_q4.cu:553-575, one with the greedy sampler behind the network and one without; the reference records a bin
  * on its first visit, inside the decode loop).  Executes nothing; the run state is untouched.  mode: REFERENCE or
  * FUSED. */
 int awq_transformer_capture(awq_transformer* t, int mode, int max_positions);
@@ -254,7 +255,9 @@ int awq_transformer_capture(awq_transformer* t, int mode, int max_positions);
 int awq_transformer_time_launches(awq_transformer* t, int passes, float* us_by_kind, int* launches_by_kind);
 
 /* run_llama_network() alone (llama2_q4.cu:430-538): the token's logits without any sampler, for callers that sample
- * on their own (the non-greedy branch of sample(), sampler.h:85-115).  mode: REFERENCE or FUSED; launched eagerly. */
+ * on their own (the non-greedy branch of sample(), sampler.h:85-115).  mode: REFERENCE or FUSED.  use_graph != 0
+ * replays a recording of the network for the position's sequence-length bin, made on first use (what run_transformer()
+ * does, llama2_q4.cu:552-590); awq_transformer_capture records those ahead of time as well. */
 int awq_transformer_forward_logits(awq_transformer* t, int use_graph, int mode);
 /* The tail of the reference's samplers (gpu_kernels.h:490-500, 582-591) for a token chosen by the caller:
  * p = pos + 1; if write_token, tokens[p] = token; pos = p (pinned-host and device copies). */

@@ -101,8 +101,10 @@ struct awq_transformer {
     // only current after the stream has drained).  Sizes the attention launch, selects the graph bin and bounds
     // the sequence; kept by reset / set_pos / forward / accept / sample / prefill.
     int issued_pos;
-    hipGraphExec_t graphs[2][kMaxGraphs];
+    hipGraphExec_t graphs[2][kMaxGraphs];      // network + greedy sampler, per schedule and sequence-length bin
     bool captured[2][kMaxGraphs];
+    hipGraphExec_t graphs_net[2][kMaxGraphs];  // the network alone (what the reference itself records, llama2_q4.cu:560-575)
+    bool captured_net[2][kMaxGraphs];
     int* tokens_dev;  // device mirror of SharedData.tokens (the persistent kernel reads its input token here)
     float2* rope_table;  // [seq_len][head_size/2] (cos, sin)
     float* attn_part;    // [kAttnMaxChunks][dim] fp32 partial attention outputs of the position-split form
@@ -224,7 +226,10 @@ void release(awq_transformer* t) {
     if (!t) return;
     for (int m = 0; m < 2; m++)
         for (int i = 0; i < kMaxGraphs; i++)
+        {
             if (t->captured[m][i]) (void)hipGraphExecDestroy(t->graphs[m][i]);
+            if (t->captured_net[m][i]) (void)hipGraphExecDestroy(t->graphs_net[m][i]);
+        }
     (void)hipFree(t->blob);
     (void)hipFree(t->s.x);
     (void)hipFree(t->s.xb);
@@ -580,15 +585,17 @@ int graph_bin(const awq_config& cfg, int seq_len, int* seq_len_bin_out) {
     return graph_index;
 }
 
-// Record and instantiate the launch sequence (network + greedy sampler) of one bin, unless that is done already.
-// Recording executes nothing and leaves the run state untouched.
-int ensure_captured(awq_transformer* t, int mode, int graph_index, int seq_len_bin) {
-    if (t->captured[mode][graph_index]) return AWQ_OK;
+// Record and instantiate the launch sequence of one bin (the network, with or without the greedy sampler behind it),
+// unless that is done already.  Recording executes nothing and leaves the run state untouched.
+int ensure_captured(awq_transformer* t, int mode, int graph_index, int seq_len_bin, bool with_sampler = true) {
+    bool* done = with_sampler ? &t->captured[mode][graph_index] : &t->captured_net[mode][graph_index];
+    hipGraphExec_t* exec = with_sampler ? &t->graphs[mode][graph_index] : &t->graphs_net[mode][graph_index];
+    if (*done) return AWQ_OK;
     awq_ctx* ctx = t->ctx;
     hipGraph_t graph = nullptr;
     AWQ_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
     int r = network(t, seq_len_bin, mode);
-    if (r == AWQ_OK)
+    if (r == AWQ_OK && with_sampler)
         r = awq_launch_argmax(ctx, t->s.logits, t->cfg.vocab_size, t->s.shared_tokens, t->s.shared_pos, t->s.pos, 1, t->tokens_dev);
     hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
     if (r) {
@@ -599,13 +606,13 @@ int ensure_captured(awq_transformer* t, int mode, int graph_index, int seq_len_b
         awq_set_error("hipStreamEndCapture failed: %s", hipGetErrorString(e));
         return AWQ_ERR_HIP;
     }
-    e = hipGraphInstantiate(&t->graphs[mode][graph_index], graph, nullptr, nullptr, 0);
+    e = hipGraphInstantiate(exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
     if (e != hipSuccess) {
         awq_set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
         return AWQ_ERR_HIP;
     }
-    t->captured[mode][graph_index] = true;
+    *done = true;
     return AWQ_OK;
 }
 
@@ -925,11 +932,17 @@ int awq_transformer_forward_logits(awq_transformer* t, int use_graph, int mode) 
     AWQ_REQUIRE(t, AWQ_ERR_ARG, "null transformer");
     AWQ_REQUIRE(mode == AWQ_SCHEDULE_REFERENCE || mode == AWQ_SCHEDULE_FUSED, AWQ_ERR_ARG,
                 "forward_logits runs the reference or the fused schedule");
-    (void)use_graph;  // the recorded sequences include the sampler; this entry point always launches eagerly
     awq_ctx* ctx = t->ctx;
     if (int r = awq_bind(ctx)) return r;
     const int seq_len = t->issued_pos + 1;
     AWQ_REQUIRE(seq_len <= t->cfg.seq_len, AWQ_ERR_ARG, "position beyond seq_len");
+    if (use_graph) {  // run_transformer(), llama2_q4.cu:552-590: the network of the position's bin, recorded on first use
+        int seq_len_bin;
+        const int graph_index = graph_bin(t->cfg, seq_len, &seq_len_bin);
+        if (int r = ensure_captured(t, mode, graph_index, seq_len_bin, false)) return r;
+        AWQ_HIP_TRY(hipGraphLaunch(t->graphs_net[mode][graph_index], ctx->stream));
+        return AWQ_OK;
+    }
     return network(t, seq_len, mode);
 }
 
@@ -1004,7 +1017,8 @@ int awq_transformer_capture(awq_transformer* t, int mode, int max_positions) {
         int seq_len_bin;
         const int graph_index = graph_bin(t->cfg, seq_len, &seq_len_bin);
         if (graph_index != last) {
-            if (int r = ensure_captured(t, mode, graph_index, seq_len_bin)) return r;
+            if (int r = ensure_captured(t, mode, graph_index, seq_len_bin, true)) return r;
+            if (int r = ensure_captured(t, mode, graph_index, seq_len_bin, false)) return r;
             last = graph_index;
         }
         seq_len = (seq_len_bin < max_positions ? seq_len_bin : max_positions);  // jump to the end of this bin
@@ -1045,13 +1059,16 @@ int awq_transformer_forward(awq_transformer* t, int gen_token, int use_graph, in
         const int graph_index = graph_bin(t->cfg, seq_len, &seq_len_bin);
         if ((r = ensure_captured(t, mode, graph_index, seq_len_bin))) return r;
         // The recorded sampler always writes its token; while the prompt is being consumed the next prompt
-        // token must survive, so those steps run eagerly below.
+        // token must survive, so those steps replay the recording of the network alone and launch the sampler
+        // (which then only advances the position) behind it.
         if (gen_token) {
             AWQ_HIP_TRY(hipGraphLaunch(t->graphs[mode][graph_index], ctx->stream));
             t->issued_pos++;
             return AWQ_OK;
         }
-        r = network(t, seq_len_bin, mode);
+        if ((r = ensure_captured(t, mode, graph_index, seq_len_bin, false))) return r;
+        AWQ_HIP_TRY(hipGraphLaunch(t->graphs_net[mode][graph_index], ctx->stream));
+        r = AWQ_OK;
     } else {
         r = network(t, seq_len, mode);
     }

@@ -41,7 +41,7 @@ def _logits(seed, n, scale):
     return (np.random.default_rng(seed).normal(0, scale, n)).astype(np.float16)
 
 
-@pytest.mark.parametrize("n,temperature,scale", [(32000, 0.5, 2.0), (32000, 1.0, 5.0), (1000, 0.7, 1.0), (5, 0.3, 1.0), (1025, 2.0, 8.0), (65535, 0.9, 3.0)])
+@pytest.mark.parametrize("n,temperature,scale", [(32000, 0.5, 2.0), (32000, 1.0, 5.0), (1000, 0.7, 1.0), (5, 0.3, 1.0), (1025, 2.0, 8.0), (65535, 0.9, 3.0), (40000, 0.7, 2.0), (32768, 0.6, 3.0), (32769, 0.6, 3.0)])
 def test_softmax_logits(ctx, n, temperature, scale):
     l = _logits(3, n, scale)
     d = ctx.upload(l.view(np.uint16))
@@ -60,16 +60,16 @@ def _oracle_pick(probs, threshold, sorted_):
 
 
 @pytest.mark.parametrize("sorted_", [0, 1])
-@pytest.mark.parametrize("case", range(8))
+@pytest.mark.parametrize("case", range(10))
 def test_sample_top_p_identical_to_oracle(ctx, case, sorted_):
     rng = np.random.default_rng(200 + case)
-    n = [32000, 32000, 4097, 777, 64, 3, 65535, 1024][case]
+    n = [32000, 32000, 4097, 777, 64, 3, 65535, 1024, 40000, 49153][case]  # up to 32768 / 49152 / 65535: three forms of the kernels
     if case == 7:
         probs = np.full(n, 1.0 / 1024, dtype=np.float16)  # all equal: pure tie-breaking by index
     elif case == 6:
         probs = oracle.softmax_logits(_logits(case, n, 0.2), 1.0)  # nearly flat: thousands of equal values per bin
     else:
-        probs = oracle.softmax_logits(_logits(case, n, [2.0, 7.0, 1.0, 3.0, 0.5, 1.0][case]), 0.8)
+        probs = oracle.softmax_logits(_logits(case, n, [2.0, 7.0, 1.0, 3.0, 0.5, 1.0, 0, 0, 2.0, 4.0][case]), 0.8)
     d = ctx.upload(probs.view(np.uint16))
     pin = Pinned(ctx)
     thresholds = list(rng.uniform(0, 1, 20)) + [0.0, 1e-8, 2.0 ** -24, 0.5, 0.999, 1.0, 1.0005, 1.5]
@@ -125,9 +125,11 @@ def test_sampler_object_follows_reference_sample(ctx, temperature, topp):
     pin.close()
 
 
-def test_transformer_sample_loop(ctx):
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_transformer_sample_loop(ctx, use_graph):
     """forward_logits + sample on a small model: greedy sampler == the fused forward; stochastic sampler picks what
-    the oracle picks from the GPU's own probabilities, and the token feeds the next step."""
+    the oracle picks from the GPU's own probabilities, and the token feeds the next step.  With use_graph the network
+    is a replayed recording (llama2_q4.cu:552-590) and the sampler is launched behind it."""
     cfg = dict(dim=256, hidden_dim=768, n_layers=2, n_heads=2, n_kv_heads=2, vocab_size=2048, seq_len=64, rope_theta=10000.0)
     img = synth.make_model_image(cfg, seed=5)
     prompt = [3, 9, 27]
@@ -137,14 +139,14 @@ def test_transformer_sample_loop(ctx):
     t.reset(prompt)
     for pos in range(12):
         ctx.sync()
-        t.forward_logits()
+        t.forward_logits(use_graph)
         t.sample(g, pos >= len(prompt) - 1)
     ctx.sync()
     greedy = [t.token(i) for i in range(13)]
     t.reset(prompt)
     for pos in range(12):
         ctx.sync()
-        t.forward(pos >= len(prompt) - 1)
+        t.forward(pos >= len(prompt) - 1, use_graph)
     ctx.sync()
     assert greedy == [t.token(i) for i in range(13)]
     g.close()
@@ -155,7 +157,7 @@ def test_transformer_sample_loop(ctx):
     t.reset(prompt)
     for pos in range(16):
         ctx.sync()
-        t.forward_logits()
+        t.forward_logits(use_graph)
         gen = pos >= len(prompt) - 1
         t.sample(s, gen)
         ctx.sync()
@@ -169,3 +171,42 @@ def test_transformer_sample_loop(ctx):
             assert t.token(pos + 1) == prompt[pos + 1]
     s.close()
     t.close()
+
+
+def test_recorded_network_equals_eager_across_bins(ctx):
+    """forward_logits as a replayed recording gives the logits of the eager launch sequence, bit for bit, on both sides
+    of the 128-position bin boundary (the recordings are keyed by bin; positions are read from device memory), and
+    prompt steps of forward(use_graph) leave the prompt's tokens alone."""
+    cfg = dict(dim=256, hidden_dim=768, n_layers=2, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=300, rope_theta=10000.0)
+    img = synth.make_model_image(cfg, seed=8)
+    prompt = [int(x) for x in synth.prompt_tokens(3, 140, cfg["vocab_size"])]
+    g = A.Sampler(ctx, cfg["vocab_size"], 0.0, 0.9, 1)
+    logits = {}
+    for use_graph in (False, True):
+        t = A.Transformer(ctx, image=img)
+        t.reset(prompt)
+        rows = []
+        for pos in range(150):
+            ctx.sync()
+            t.forward_logits(use_graph)
+            ctx.sync()
+            if pos in (0, 5, 126, 127, 128, 129, 140, 149):
+                rows.append(t.download("logits", cfg["vocab_size"]).copy())
+            t.sample(g, pos >= len(prompt) - 1)
+        ctx.sync()
+        logits[use_graph] = (rows, [t.token(i) for i in range(151)])
+        t.close()
+    for a, b in zip(logits[False][0], logits[True][0]):
+        assert np.array_equal(a, b)
+    assert logits[False][1] == logits[True][1]
+    assert logits[True][1][: len(prompt)] == prompt
+    # forward(use_graph) through the prompt: recorded network + sampler that only advances
+    t = A.Transformer(ctx, image=img)
+    t.reset(prompt)
+    for pos in range(150):
+        ctx.sync()
+        t.forward(pos >= len(prompt) - 1, True)
+    ctx.sync()
+    assert [t.token(i) for i in range(151)] == logits[False][1]
+    t.close()
+    g.close()
