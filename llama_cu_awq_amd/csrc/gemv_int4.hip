@@ -37,6 +37,7 @@ struct GemvParams {
     const uint16_t* norm_w;  // RMSNorm weights when the norm is fused into staging
     uint16_t* norm_out;      // optional: block 0 also stores the normalised vector here
     int K, N;
+    int Nkv;                 // QKV form: rows of the K and V matrices (grouped-query models have fewer than N); else = N
     int C;                   // 32-element chunks per row = ceil(K/32)
     int pzh, sh;             // zeros dwords / scale halves per row
     int accum;
@@ -104,6 +105,9 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     const int P = (int)(((uint32_t)C + LPR - 1) / LPR);  // passes per row (per SPLIT rows)
     float* ca = reinterpret_cast<float*>(xs + 4 * C);
     const int which = (KIND == KIND_QKV) ? blockIdx.y : 0;
+    const int N = (KIND == KIND_QKV && which != 0) ? p.Nkv : p.N;  // rows of this workgroup's matrix
+    // (the grid is sized for the Q matrix; workgroups beyond the K and V rows of a grouped-query model have nothing to do)
+    if (KIND == KIND_QKV && (int)blockIdx.x * (W * SPLIT * R) >= N) return;
     const bool rope_here = ROPE && which != 2;
     constexpr bool RES = KIND == KIND_SINGLE;
 
@@ -148,10 +152,10 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
     auto set_rows = [&](int g) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const int li = min((g * W + wave) * RW + SPLIT * r, p.N - 1);  // indices past N are recomputed, never stored
+            const int li = min((g * W + wave) * RW + SPLIT * r, N - 1);  // indices past N are recomputed, never stored
             const int row = rope_here ? map_row<true>(li, p.half_shift) : li;
             if (HALF) {
-                const int li_own = min((g * W + wave) * RW + SPLIT * r + hf, p.N - 1);
+                const int li_own = min((g * W + wave) * RW + SPLIT * r + hf, N - 1);
                 const int drow = (rope_here ? map_row<true>(li_own, p.half_shift) : li_own) - row;
                 hoff_w[r] = (uint32_t)drow * p.wbytes;
                 hoff_z[r] = (uint32_t)drow * p.zbytes;
@@ -232,15 +236,15 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
                 second[r] = 0.0f;
                 if (HALF) second[r] = __shfl_xor(sum[r], LPR);
             }
-            if (ll == 0 && (hf & 1) == 0 && li0 + hf < p.N) {
+            if (ll == 0 && (hf & 1) == 0 && li0 + hf < N) {
                 uint16_t* out = out_base;
-                if (loff != -1) out += (size_t)loff + (size_t)pos_now * p.N;
+                if (loff != -1) out += (size_t)loff + (size_t)pos_now * N;
                 const int half = p.head_size >> 1;
                 const float2* cs_tab = p.rope + (size_t)pos_now * half;
 #pragma unroll
                 for (int r = 0; r < (HALF ? R : R - 1); r += (HALF ? 1 : 2)) {
                     const int li = li0 + (HALF ? SPLIT * r + hf : r);
-                    if (li < p.N) {
+                    if (li < N) {
                         const int row = map_row<true>(li, p.half_shift);
                         const float v0 = half_bits_to_float(float_to_half_bits(sum[r]));
                         const float v1 = half_bits_to_float(float_to_half_bits(HALF ? second[r] : sum[HALF ? r : r + 1]));
@@ -254,11 +258,11 @@ __global__ __launch_bounds__(W * 64) void gemv_int4_kernel(const GemvParams p) {
             }
         } else if (ll == 0) {
             uint16_t* out = out_base;
-            if (loff != -1) out += (size_t)loff + (size_t)pos_now * p.N;
+            if (loff != -1) out += (size_t)loff + (size_t)pos_now * N;
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 const int row = li0 + (HALF ? SPLIT * r + hf : r);
-                if (row < p.N) {
+                if (row < N) {
                     float v;
                     if (KIND == KIND_FFN) {
                         // gate = stream 2r, up = stream 2r+1 (gpu_kernels.h:276-281)
@@ -400,6 +404,7 @@ void fill_common(GemvParams& p, const uint16_t* x, int K, int N) {
     p.norm_out = nullptr;
     p.K = K;
     p.N = N;
+    p.Nkv = N;
     p.C = div_up(K, 32);
     p.pzh = packed_zeros_height(K);
     p.sh = scales_height(K);
@@ -579,7 +584,7 @@ int dispatch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what, GemvPlan
                 // compute unit, so three on some) or 501 of 10 (two on each): 16.5 -> 16.1 us, +0.75 % tokens/s at the
                 // 33B shape
                 auto unevenness = [&](int w) {
-                    const double per_cu = (double)div_up(p.N, w * 4) * grid_y / ctx->cus;
+                    const double per_cu = (double)(div_up(p.N, w * 4) + (grid_y - 1) * div_up(p.Nkv, w * 4)) / ctx->cus;
                     return ceil(per_cu) / per_cu;
                 };
                 if (unevenness(10) < unevenness(8) - 0.15) return dispatch_split<10, KIND, ROPE, 4>(ctx, p, grid_y, what, depth);
@@ -638,9 +643,10 @@ int awq_launch_matvec_int4_parts(awq_ctx* ctx, uint16_t* out, const float* part,
 
 int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
                    const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw, int K, int N, int loff,
-                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out, const float2* rope, int head_size) {
+                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out, const float2* rope, int head_size, int Nkv) {
     GemvParams p;
     fill_common(p, x, K, N);
+    p.Nkv = Nkv;  // = N in the reference's qkv_matvec_kernel (llama2_q4.cu:454); fewer rows in grouped-query models
     p.rope = rope;
     p.head_size = head_size;
     p.m[0] = to_mat(qw);
@@ -703,7 +709,7 @@ int awq_qkv_matvec(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* val
     if (int r = check_shape(K, N)) return r;
     AWQ_REQUIRE(q && key_cache && value_cache && x && qw_ok(qw) && qw_ok(kw) && qw_ok(vw), AWQ_ERR_ARG, "null pointer");
     AWQ_REQUIRE(loff >= 0 && pos, AWQ_ERR_ARG, "qkv needs loff >= 0 and a position pointer");
-    return awq_launch_qkv(ctx, q, key_cache, value_cache, x, qw, kw, vw, K, N, loff, pos, nullptr, nullptr, nullptr, 0);
+    return awq_launch_qkv(ctx, q, key_cache, value_cache, x, qw, kw, vw, K, N, loff, pos, nullptr, nullptr, nullptr, 0, N);
 }
 
 int awq_ffn_matvec_silu(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w, const awq_qweight* up_w,

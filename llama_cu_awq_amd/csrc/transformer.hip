@@ -18,7 +18,7 @@ int awq_launch_matvec_int4(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const
                            int gpu_count, int loff, const int* pos, const uint16_t* norm_w, uint16_t* norm_out);
 int awq_launch_qkv(awq_ctx* ctx, uint16_t* q, uint16_t* key_cache, uint16_t* value_cache, const uint16_t* x,
                    const awq_qweight* qw, const awq_qweight* kw, const awq_qweight* vw, int K, int N, int loff,
-                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out, const float2* rope, int head_size);
+                   const int* pos, const uint16_t* norm_w, uint16_t* norm_out, const float2* rope, int head_size, int Nkv);
 int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qweight* gate_w, const awq_qweight* up_w, int K,
                    int N, const uint16_t* norm_w, uint16_t* norm_out);
 int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
@@ -515,21 +515,12 @@ int network_fused(awq_transformer* t, int seq_len_bin) {
         const int loff = l * p.seq_len * kv_dim;
         {
             LaunchProbe probe(t, LK_QKV);
-            if (dim == kv_dim) {
-                if ((r = awq_launch_qkv(ctx, s.q, s.key_cache, s.value_cache, s.x, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, loff, pPos,
-                                        L.rms_att_weight, nullptr, t->rope_table, head_size)))
-                    return r;
-            } else {
-                if ((r = awq_launch_matvec_int4(ctx, s.q, s.x, &L.wq_q, dim, dim, 0, 1, -1, nullptr, L.rms_att_weight, nullptr)))
-                    return r;
-                if ((r = awq_launch_matvec_int4(ctx, s.key_cache, s.x, &L.wq_k, dim, kv_dim, 0, 1, loff, pPos, L.rms_att_weight,
-                                                nullptr)))
-                    return r;
-                if ((r = awq_launch_matvec_int4(ctx, s.value_cache, s.x, &L.wq_v, dim, kv_dim, 0, 1, loff, pPos, L.rms_att_weight,
-                                                nullptr)))
-                    return r;
-                if ((r = awq_rope(ctx, s.q, s.key_cache, p.n_heads, p.n_kv_heads, head_size, pPos, loff, p.rope_theta))) return r;
-            }
+            // one launch for the three matrices, RMSNorm in its staging and the rotation in its epilogue; with grouped
+            // queries (the reference then makes three launches and the rotation, llama2_q4.cu:457-464) the K and V
+            // matrices have kv_dim rows and the workgroups past them leave at once
+            if ((r = awq_launch_qkv(ctx, s.q, s.key_cache, s.value_cache, s.x, &L.wq_q, &L.wq_k, &L.wq_v, dim, dim, loff, pPos,
+                                    L.rms_att_weight, nullptr, t->rope_table, head_size, kv_dim)))
+                return r;
         }
         // Long launch sizes: P.V split over positions too, its fp32 partial sums added up (and rounded to fp16, the
         // reference's rounding point) while the O projection stages its input; xb is not written on this path.
