@@ -7,7 +7,8 @@ real layout and distributions, resident in HBM before the timed region starts.
 
 Prints ONE JSON line: tokens/s (`value`) of the run the flags ask for; `config1`, the benchmark's own run (16-token
 prompt + 256 decode steps from position 0) whatever the flags were; `config2` and `config3`, 256 decode steps of the 13B
-shape from a KV cache pre-filled to position 1536 and of the 33B shape; the roofline of the dominant kernel as the timed
+shape from a KV cache pre-filled to position 1536 and of the 33B shape; `shape_70b`, 128 steps of Llama-2-70B's shape
+(grouped queries, 36.6 GB packed; not one of the benchmark's configurations); the roofline of the dominant kernel as the timed
 schedule launches it (RMSNorm-fused gate/up int4 matrix-vector product, timed live with HIP events over the 32
 layers' distinct weights); `config0`, the single 4096 x 4096 product back to back on one stream and dealt over 2 and 4
 plain streams; the 512-token prefill; and the CPU oracle timed on a bounded sample of the same workload.
@@ -79,8 +80,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--config", default="7b", choices=["7b", "13b", "33b"])
-    ap.add_argument("--scale-mult", type=float, default=None, help="multiplies the weights' scale range U[0.002, 0.02]; default 1.0, and 0.5 for --config 33b (60 layers leave fp16 range at 1.0)")
+    ap.add_argument("--config", default="7b", choices=["7b", "13b", "33b", "70b"])
+    ap.add_argument("--scale-mult", type=float, default=None, help="multiplies the weights' scale range U[0.002, 0.02]; default 1.0, 0.5 for --config 33b and 0.25 for 70b (60 and 80 layers leave fp16 range at 1.0)")
     ap.add_argument("--start-pos", type=int, default=0, help="pre-fill the KV cache with N(0,1) up to this position first")
     ap.add_argument("--schedule", default="fused", choices=["persistent", "fused", "reference"])
     ap.add_argument("--no-graph", action="store_true")
@@ -99,7 +100,7 @@ def main():
     import llama_cu_awq_amd as A
     from llama_cu_awq_amd import synth
 
-    cfg = {"7b": synth.CONFIG_7B, "13b": synth.CONFIG_13B, "33b": synth.CONFIG_33B}[args.config]
+    cfg = {"7b": synth.CONFIG_7B, "13b": synth.CONFIG_13B, "33b": synth.CONFIG_33B, "70b": synth.CONFIG_70B}[args.config]
     n_prompt = max(1, args.warmup)
     total = n_prompt + args.steps
     assert args.start_pos + total <= cfg["seq_len"], "warmup + steps exceeds seq_len"
@@ -107,7 +108,7 @@ def main():
     use_graph = not args.no_graph
 
     t0 = time.time()
-    scale_mult = args.scale_mult if args.scale_mult is not None else (0.5 if args.config == "33b" else 1.0)
+    scale_mult = args.scale_mult if args.scale_mult is not None else {"33b": 0.5, "70b": 0.25}.get(args.config, 1.0)
     image = synth.make_model_image(cfg, seed=args.seed, threads=min(16, os.cpu_count() or 8), scale_mult=scale_mult)
     print(f"[bench] model image {image.nbytes / 1e9:.2f} GB generated in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
     ctx = A.Context(0)
@@ -338,8 +339,8 @@ def main():
         model.close()
         model = None
         del image
-        for key, name, start, steps, scale in (("config2", "13b", 1536, 256, 1.0), ("config3", "33b", 0, 256, 0.5)):
-            xcfg = {"13b": synth.CONFIG_13B, "33b": synth.CONFIG_33B}[name]
+        for key, name, start, steps, scale in (("config2", "13b", 1536, 256, 1.0), ("config3", "33b", 0, 256, 0.5), ("shape_70b", "70b", 0, 128, 0.25)):
+            xcfg = {"13b": synth.CONFIG_13B, "33b": synth.CONFIG_33B, "70b": synth.CONFIG_70B}[name]
             t0 = time.time()
             ximg = synth.make_model_image(xcfg, seed=args.seed, threads=min(16, os.cpu_count() or 8), scale_mult=scale)
             xm = A.Transformer(ctx, image=ximg)

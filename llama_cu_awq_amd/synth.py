@@ -203,3 +203,5 @@ def prompt_tokens(seed, n, vocab):
 CONFIG_7B = dict(dim=4096, hidden_dim=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab_size=32000, seq_len=2048, rope_theta=10000.0)
 CONFIG_13B = dict(dim=5120, hidden_dim=13824, n_layers=40, n_heads=40, n_kv_heads=40, vocab_size=32000, seq_len=2048, rope_theta=10000.0)
 CONFIG_33B = dict(dim=6656, hidden_dim=17920, n_layers=60, n_heads=52, n_kv_heads=52, vocab_size=32000, seq_len=2048, rope_theta=10000.0)
+# beyond the benchmark's configurations: Llama-2-70B's shape (grouped queries: 64 heads share 8 KV heads), 36.6 GB packed
+CONFIG_70B = dict(dim=8192, hidden_dim=28672, n_layers=80, n_heads=64, n_kv_heads=8, vocab_size=32000, seq_len=2048, rope_theta=10000.0)

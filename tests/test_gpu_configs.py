@@ -433,6 +433,30 @@ def test_33b_shape_four_layers_matches_oracle(ctx):
         o.close()
 
 
+def test_70b_shape_grouped_queries_four_layers_matches_oracle(ctx):
+    """Llama-2-70B's layer shape (dim 8192, hidden 28672, 64 heads sharing 8 KV heads), four layers: the grouped-query
+    branch of the reference's schedule (llama2_q4.cu:457-464) against the single fused launch, rows of 28672 elements in
+    the down projection, and attention heads that share their key and value rows."""
+    cfg = dict(dim=8192, hidden_dim=28672, n_layers=4, n_heads=64, n_kv_heads=8, vocab_size=32000, seq_len=256, rope_theta=10000.0)
+    img = synth.make_model_image(cfg, seed=70, threads=THREADS, scale_mult=0.35)
+    t = A.Transformer(ctx, image=img)
+    o = oracle.Model(img)
+    try:
+        n_prompt, steps = 6, 6 + 14
+        prompt = synth.prompt_tokens(70, n_prompt, cfg["vocab_size"])
+        o.reset(prompt)
+        ref = _oracle_record(o, n_prompt, steps)
+        assert all(np.isfinite(l.astype(np.float32)).all() for l, _ in ref)
+        for mode, graph in ((A.SCHEDULE_FUSED, True), (A.SCHEDULE_REFERENCE, False)):
+            t.reset(prompt)
+            _, errs, ties = _gpu_record(t, n_prompt, steps, graph, mode, ref=ref)
+            assert max(errs) <= 1e-2, (mode, graph, max(errs))
+            assert ties <= 4, ties
+    finally:
+        t.close()
+        o.close()
+
+
 def test_33b_full_model_schedules_agree_and_stay_finite(ctx):
     """All 60 layers (17.5 GB of weights on the one GPU): the oracle would need minutes, so the check is that the two
     multi-kernel schedules, which share no matrix-vector launch geometry for the norm-fused steps, produce the same
