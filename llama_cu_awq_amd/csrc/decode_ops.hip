@@ -502,6 +502,9 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* x, int siz
     __shared__ float red_v[16];
     __shared__ int red_i[16];
     const int tid = threadIdx.x;
+    // (requested with the logits, so that it has arrived when the last thread standing needs it)
+    int token_pos = 0;
+    if (tid == 0) token_pos = *pPosGpu;
     float best = -INFINITY;
     int best_i = 0x7FFFFFFF;
     auto take = [&](float v, int i) {
@@ -552,7 +555,6 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* x, int siz
             }
         }
         if (best_i == 0x7FFFFFFF) best_i = 0;  // nothing compared greater than -inf (all NaN / -inf)
-        int token_pos = *pPosGpu;
         token_pos++;
         if (write_token) {
             result[token_pos] = best_i;

@@ -227,9 +227,9 @@ struct SampleOut {
 
 // p = position + 1; tokens[p] = idx; both copies of the position = p (the tail of sample_top_p_kernel,
 // gpu_kernels.h:585-590).  The position is read from its device copy: the two are equal, and the pinned one is a trip
-// over the host link away.
-__device__ __forceinline__ void write_token(const SampleOut& out, int idx) {
-    int token_pos = *out.pPosGpu;
+// over the host link away; the callers request it at their start (read_position), long before it is needed.
+__device__ __forceinline__ int read_position(const SampleOut& out) { return threadIdx.x == 0 ? *out.pPosGpu : 0; }
+__device__ __forceinline__ void write_token(const SampleOut& out, int idx, int token_pos) {
     token_pos++;
     out.result[token_pos] = idx;
     if (out.mirror) out.mirror[token_pos] = idx;
@@ -244,6 +244,7 @@ __device__ __forceinline__ void select_in_index_order(const uint16_t* probs, int
     __shared__ int s_best_thread;
     __shared__ int s_index;
     const int tid = threadIdx.x;
+    const int token_pos = read_position(out);
     if (tid == 0) {
         s_best_thread = kSampleThreads;
         s_index = -1;
@@ -273,7 +274,7 @@ __device__ __forceinline__ void select_in_index_order(const uint16_t* probs, int
         }
     }
     __syncthreads();
-    if (tid == 0) write_token(out, s_index >= 0 ? s_index : n - 1);
+    if (tid == 0) write_token(out, s_index >= 0 ? s_index : n - 1, token_pos);
 }
 
 // sampler.h:94-107 + gpu_kernels.h:562-592, top-p: position in the descending stable order of the probabilities at
@@ -288,7 +289,10 @@ __device__ __forceinline__ void select_in_sorted_order(const Rows<NR>& x, int n,
     __shared__ int s_bin;
     __shared__ unsigned int s_rank;
     __shared__ int s_index;
+    __shared__ int s_hi;
+    __shared__ unsigned long long s_start;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int token_pos = read_position(out);
     if (tid == 0) {
         s_best_thread = kSampleThreads;
         s_index = -1;
@@ -327,34 +331,52 @@ __device__ __forceinline__ void select_in_sorted_order(const Rows<NR>& x, int n,
     {
         // The first bin (in descending order) that holds a value and whose rounded prefix reaches the threshold lies in
         // the first thread that holds a value and whose prefix at the end of its run does (the prefix only grows, and
-        // rounding is monotone); only that thread walks its bins.
+        // rounding is monotone).
         const unsigned long long start = block_exclusive_scan_1024(total, wave_totals);
         const bool crosses = present != 0u && units_to_half_value(start + total) >= threshold;
         if (crosses) atomicMin(&s_best_thread, tid);
         __syncthreads();
         if (crosses && s_best_thread == tid) {
-            int found = -1;
-            unsigned long long before = 0, run = start;
-            for (int b = hi; b >= lo && b >= 0 && found < 0; b--) {
-                const unsigned long long add = (unsigned long long)hcount(b) * prob_units((uint32_t)b);
-                if (hcount(b) && units_to_half_value(run + add) >= threshold) {
-                    found = b;
-                    before = run;
-                }
-                run += add;
+            s_hi = hi;
+            s_start = start;
+        }
+        __syncthreads();
+        if (s_best_thread < kSampleThreads && wave == 0) {
+            // The first wave looks at that thread's bins side by side: lane j at bin s_hi - j.
+            static_assert(BPT <= 64, "a thread's bins fit the lanes of a wave");
+            const int b = s_hi - lane;
+            const bool valid = lane < BPT && b >= 0;
+            const unsigned int c = valid ? hcount(b) : 0u;
+            const unsigned long long add = (unsigned long long)c * prob_units((uint32_t)max(b, 0));
+            unsigned long long inc = add;  // inclusive prefix over the lanes (descending bins)
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const unsigned long long o = __shfl_up(inc, off);
+                if (lane >= off) inc += o;
             }
-            // how many equal values into the bin the prefix first reaches the threshold (monotone: binary search)
+            const unsigned long long hits = __ballot(c != 0u && units_to_half_value(s_start + inc) >= threshold);
+            const int first = __ffsll((long long)hits) - 1;  // some lane hits: the thread's last value crosses
+            const int found = s_hi - first;
+            const unsigned long long before = s_start + __shfl(inc - add, first);
+            const unsigned int cnt = __shfl(c, first);
+            // How many equal values into the bin the prefix first reaches the threshold: the smallest a in [1, cnt] with
+            // rounded(before + a val) >= threshold (monotone; true at a = cnt), found 64 candidates at a time.
             const unsigned long long val = prob_units((uint32_t)found);
-            unsigned int a = 1, c = hcount(found);
-            while (a < c) {
-                const unsigned int mid = (a + c) >> 1;
-                if (units_to_half_value(before + (unsigned long long)mid * val) >= threshold)
-                    c = mid;
-                else
-                    a = mid + 1;
+            unsigned int a_lo = 1, a_hi = cnt;
+            while (a_lo < a_hi) {
+                const unsigned int step = (a_hi - a_lo) / 64u + 1u;
+                const unsigned int mine = min(a_lo + (unsigned int)(lane + 1) * step - 1u, a_hi);  // lane 63 reaches a_hi
+                const unsigned long long t = __ballot(units_to_half_value(before + (unsigned long long)mine * val) >= threshold);
+                const int f = __ffsll((long long)t) - 1;
+                const unsigned int upper = __shfl(mine, f);
+                const unsigned int below = f == 0 ? a_lo : __shfl(mine, max(f - 1, 0)) + 1u;
+                a_lo = below;
+                a_hi = upper;
             }
-            s_bin = found;
-            s_rank = a;  // 1-based occurrence, in index order
+            if (lane == 0) {
+                s_bin = found;
+                s_rank = a_lo;  // 1-based occurrence, in index order
+            }
         }
     }
     __syncthreads();
@@ -399,7 +421,7 @@ __device__ __forceinline__ void select_in_sorted_order(const Rows<NR>& x, int n,
         }
     }
     __syncthreads();
-    if (tid == 0) write_token(out, s_index >= 0 ? s_index : n - 1);
+    if (tid == 0) write_token(out, s_index >= 0 ? s_index : n - 1, token_pos);
 }
 
 template <int NR>
