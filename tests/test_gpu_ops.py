@@ -392,7 +392,8 @@ def test_rope(ctx, heads, kv_heads, head, pos):
 @pytest.mark.parametrize(
     "heads,head,kv_mul,pos,max_seq",
     [(32, 128, 1, 0, 1), (32, 128, 1, 16, 17), (32, 128, 1, 271, 512), (40, 128, 1, 1791, 2048), (8, 64, 4, 300, 301), (4, 256, 2, 1023, 1024), (52, 128, 1, 2047, 2048), (8, 128, 2, 2500, 4096), (8, 64, 4, 700, 1024),
-     (8, 128, 2, 9000, 16384)],  # beyond the reference's 8192-position shared-memory form (gpu_kernels.h:411-454)
+     (8, 128, 2, 9000, 16384),  # beyond the reference's 8192-position shared-memory form (gpu_kernels.h:411-454)
+     (64, 128, 8, 300, 512)],
 )
 def test_attention(ctx, heads, head, kv_mul, pos, max_seq):
     kv_dim = heads * head // kv_mul
@@ -429,7 +430,7 @@ def test_attention(ctx, heads, head, kv_mul, pos, max_seq):
 @pytest.mark.parametrize(
     "heads,head,kv_mul,pos,max_seq",
     [(32, 128, 1, 256, 257), (32, 128, 1, 271, 512), (40, 128, 1, 1791, 2048), (52, 128, 1, 2047, 2048), (8, 64, 4, 300, 512), (4, 256, 2, 1023, 1024), (32, 128, 1, 2, 512),
-     (8, 128, 2, 9000, 16384)],
+     (8, 128, 2, 9000, 16384), (64, 128, 8, 1500, 2048)],  # the last: Llama-2-70B's heads (8 share a KV head), K = 8192 into the O projection
 )
 def test_attention_split_over_positions_then_o_projection(ctx, heads, head, kv_mul, pos, max_seq):
     """The long-context form of the fused schedule: P.V as fp32 partial sums per range of positions, added up and
