@@ -64,6 +64,55 @@ def test_matvec_int4_plain(ctx, K, N):
         assert (got != best).mean() <= max(2 * (f16(want) != best).mean(), 4e-3)
 
 
+# ---- shapes chosen to reach every branch of the launch geometry (waves per workgroup 4 / 8 / 10 / 13 / 16, one, two or
+# four rows side by side in a wave, two or three passes in flight, partly filled last workgroups and row groups, row
+# lengths that are no multiple of a pass or of a quantisation group), in the three forms.
+SWEEP_K = [8, 96, 136, 256, 512, 544, 1000, 2560, 2592, 3072, 4096, 5120, 6144, 6656, 8192, 8224, 10240, 11008, 13824, 17920, 20480,
+           28672]
+SWEEP_N = [8, 40, 264, 1000]
+
+
+@pytest.mark.parametrize("K", SWEEP_K)
+def test_matvec_int4_shape_sweep(ctx, K):
+    for N in SWEEP_N + ([5120] if K in (5120, 13824) else []) + ([6656] if K in (6656, 17920) else []):
+        w, z, s, x = _case(K, N, 7)
+        truth = synth.dequantize(w, z, s, K) @ x.astype(np.float64)
+        qw = A.QWeight.upload(ctx, w, z, s)
+        dx = ctx.upload(x)
+        # single matrix, with the residual added
+        resid = synth.normal_f16(synth.stream_key(7, "res", K, N), N)
+        dout = ctx.upload(resid)
+        A.matmul_q(ctx, dout, dx, qw, K, N, accum=True)
+        got = f16(dout.download(np.uint16))
+        want = resid.view(np.uint16).copy()
+        oracle.matvec_int4(want, x, w, z, s, K, N, accum=True)
+        assert_close_f16(got, f16(want), ulps=2)
+        assert rel_l2(got, truth + resid.astype(np.float64)) <= 1e-3, ("single", K, N)
+        # the three-matrix form (the same matrix three times: q, and one row each of the two caches)
+        pos, loff, rows = 1, N, 3
+        dq, dk, dv = ctx.zeros(N * 2), ctx.zeros(rows * N * 2), ctx.zeros(rows * N * 2)
+        dpos = ctx.upload(np.array([pos], dtype=np.int32))
+        A.qkv_matvec(ctx, dq, dk, dv, dx, qw, qw, qw, K, N, loff, dpos)
+        plain = np.zeros(N, dtype=np.uint16)
+        oracle.matvec_int4(plain, x, w, z, s, K, N)
+        for buf, off in ((dq, 0), (dk, loff + pos * N), (dv, loff + pos * N)):
+            g = buf.download(np.uint16)
+            assert_close_f16(f16(g[off : off + N]), f16(plain), ulps=2)
+            assert not g[:off].any() and not g[off + N :].any(), ("qkv", K, N)
+        # gate/up with SiLU (the matrix against a second one)
+        w2, z2, s2, _ = _case(K, N, 8)
+        qw2 = A.QWeight.upload(ctx, w2, z2, s2)
+        xs = (x.astype(np.float32) * np.float32(0.25)).astype(np.float16)  # keeps SiLU(g) * u inside fp16 at the long rows
+        dh = ctx.zeros(N * 2)
+        A.ffn_matvec_silu(ctx, dh, ctx.upload(xs), qw, qw2, K, N)
+        hw = np.zeros(N, dtype=np.uint16)
+        oracle.ffn_matvec_silu(hw, xs, (w, z, s), (w2, z2, s2), K, N)
+        gh, hw = f16(dh.download(np.uint16)), f16(hw)
+        assert np.isfinite(hw.astype(np.float32)).all()
+        assert rel_l2(gh, hw) <= 1e-3, ("ffn", K, N)
+        assert_close_f16(gh, hw, ulps=4)
+
+
 # ---- activations far from unit magnitude.  The reference multiplies (q - z) * s * x in fp32 whatever the size of x
 # (gpu_kernels.h:203-207), so a vector that is small as a whole (the attention output in front of the O projection,
 # SiLU(gate) * up in front of the down projection) must come out as accurately as a vector of order one.  The scaled
@@ -262,7 +311,7 @@ def test_qkv_matvec(ctx, K, N):
     assert rel_l2(f16(kgot[loff + pos * N : loff + (pos + 1) * N]), truth) <= 1e-3
 
 
-@pytest.mark.parametrize("K,N", [(4096, 11008), (5120, 13824), (6656, 17920), (256, 72), (1024, 4480)])
+@pytest.mark.parametrize("K,N", [(4096, 11008), (5120, 13824), (6656, 17920), (256, 72), (1024, 4480), (8192, 1024), (2560, 264), (136, 40), (10240, 520)])
 def test_rmsnorm_ffn_matvec_silu_equals_the_two_calls(ctx, K, N):
     """The one-launch form of rmsnorm + ffn_matvec_silu (what the fused schedule runs) against the oracle's two steps:
     the normalised vector must be the same fp16 values, so the outputs agree as closely as the plain kernel's do."""
