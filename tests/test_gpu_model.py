@@ -76,6 +76,53 @@ def test_greedy_decode_matches_oracle(pair, mode, graph):
     assert worst <= 1e-2, worst
 
 
+# Shapes that send the fused schedule's QKV launch (RMSNorm and rotation inside; reachable through the model only) down
+# its different forms: rows of 2.5 and 1.25 passes of 64 lanes (two and four rows side by side in a wave), of less than
+# one pass, grouped queries with each of those, and the three head sizes.
+SHAPES_FUSED = {
+    "rows-of-2560": dict(dim=2560, hidden_dim=3456, n_layers=1, n_heads=20, n_kv_heads=20),
+    "rows-of-2560-grouped": dict(dim=2560, hidden_dim=3456, n_layers=2, n_heads=20, n_kv_heads=4),
+    "rows-of-640": dict(dim=640, hidden_dim=1728, n_layers=2, n_heads=5, n_kv_heads=5),
+    "rows-of-640-grouped": dict(dim=640, hidden_dim=1728, n_layers=2, n_heads=5, n_kv_heads=1),
+    "rows-of-1280": dict(dim=1280, hidden_dim=3456, n_layers=1, n_heads=10, n_kv_heads=2),
+    "heads-of-64": dict(dim=320, hidden_dim=864, n_layers=2, n_heads=5, n_kv_heads=5),
+    "heads-of-256": dict(dim=768, hidden_dim=2048, n_layers=2, n_heads=3, n_kv_heads=1),
+}
+
+
+@pytest.mark.parametrize("shape", sorted(SHAPES_FUSED))
+def test_model_shapes_through_the_fused_schedule(ctx, shape):
+    cfg = dict(SHAPES_FUSED[shape], vocab_size=512, seq_len=40, rope_theta=10000.0)
+    img = synth.make_model_image(cfg, seed=11, scale_mult=0.5)
+    t = A.Transformer(ctx, image=img)
+    o = oracle.Model(img)
+    try:
+        prompt = synth.prompt_tokens(4, 5, cfg["vocab_size"])
+        kv_dim = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"]
+        for mode, graph in ((A.SCHEDULE_FUSED, False), (A.SCHEDULE_FUSED, True), (A.SCHEDULE_REFERENCE, False)):
+            t.reset(prompt)
+            o.reset(prompt)
+            for step in range(12):
+                t.ctx.sync()
+                gen = step >= len(prompt) - 1
+                t.forward(gen_token=gen, use_graph=graph, mode=mode)
+                o.forward(gen_token=gen)
+                t.ctx.sync()
+                got, want = f16(t.download("logits", cfg["vocab_size"])), f16(o.buffer("logits", cfg["vocab_size"]))
+                assert rel_l2(got, want) <= 1e-2, (shape, mode, graph, step)
+                if t.token(step + 1) != o.tokens(step + 2)[step + 1]:  # a flip on a near tie: follow the oracle
+                    top = np.sort(want.astype(np.float64))
+                    assert top[-1] - top[-2] <= 4 * np.abs(got.astype(np.float64) - want.astype(np.float64)).max(), (shape, step)
+                    t.set_pos(step + 1, o.tokens(step + 2)[step + 1])
+            n = 12 * kv_dim
+            for name in ("key_cache", "value_cache"):
+                assert rel_l2(f16(t.download(name, n)), f16(o.buffer(name, n))) <= 1e-2, (shape, mode, name)
+            assert rel_l2(f16(t.download("q", cfg["dim"])), f16(o.buffer("q", cfg["dim"]))) <= 1e-2
+    finally:
+        t.close()
+        o.close()
+
+
 def test_capture_ahead_of_time_changes_nothing(ctx):
     """Recording every bin up front (seq_len 300: bins 128, 256 and the model's own length) leaves the run state alone
     and gives the tokens of a run that records on first visit; the bins are crossed inside the run."""
