@@ -216,6 +216,23 @@ def main():
     model.set_pos(min(mid, cfg["seq_len"] - 1), prompt[0])
     in_place = model.time_launches(passes=4)
     ffn_us = in_place["gate_up"]["us"]
+    # every launch kind of the fused schedule against the HBM roofline: algorithmic bytes per launch (packed weights,
+    # activations in and out, norm weights; attention: the key and value rows up to the position) over its time in place
+    kv_rows_bytes = 2 * (min(mid, cfg["seq_len"] - 1) + 1) * kv_dim * 2
+    launch_bytes = {
+        "embed": 2 * dim * 2,
+        "qkv": qweight_bytes(dim, dim) + 2 * qweight_bytes(dim, kv_dim) + 2 * dim * 2 + (dim + 2 * kv_dim) * 2,
+        "attention": kv_rows_bytes + 2 * dim * 2,
+        "oproj": qweight_bytes(dim, dim) + 3 * dim * 2,
+        "gate_up": 2 * qweight_bytes(dim, hid) + 2 * dim * 2 + hid * 2,
+        "down": qweight_bytes(hid, dim) + hid * 2 + 2 * dim * 2,
+        "classifier": vocab * dim * 2 + 2 * dim * 2 + vocab * 2,
+    }
+    launch_table = {
+        k: {"us": v["us"], "bytes": launch_bytes[k], "gbps": round(launch_bytes[k] / v["us"] / 1e3, 1) if v["us"] else None,
+            "frac_of_hbm_peak": round(launch_bytes[k] / v["us"] / 1e3 / (HBM_PEAK / 1e9), 4) if v["us"] else None}
+        for k, v in in_place.items()
+    }
     ffn_bytes = 2 * qweight_bytes(dim, hid) + dim * 2 + dim * 2 + hid * 2  # weights, x, norm weights, out
     ffn_gbps = ffn_bytes / ffn_us / 1e3
     ffn_waves = 4 if dim <= 8192 else 16
@@ -418,6 +435,7 @@ def main():
             "first_tokens": gen,
         },
         "launches_in_place_us": {k: v["us"] for k, v in in_place.items()},
+        "launches_in_place": launch_table,
         "config0": config0,
         "config1": config1,
     }
