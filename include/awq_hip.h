@@ -273,7 +273,8 @@ int awq_softmax_logits(awq_ctx* ctx, uint16_t* logits, int size, float temperatu
  * index order; the token is the first position whose inclusive prefix sum, rounded to fp16, is >= threshold
  * (position size-1 when none is).  The prefix sums are exact (fp16 values are multiples of 2^-24) and rounded once;
  * the reference's CUB scan adds in fp16 in an unspecified order.  Then p = pos + 1; tokens[p] = token; pos = p
- * (pinned-host and device copies).  probs is left untouched.  size <= 65535. */
+ * (pinned-host and device copies).  probs is left untouched.  size <= 1048576 (above 65535 entries a slower,
+ * plain form of the kernels runs). */
 int awq_sample_top_p(awq_ctx* ctx, const uint16_t* probs, int size, float threshold, int sorted, int* tokens,
                      volatile int* pos_host, int* pos_dev);
 

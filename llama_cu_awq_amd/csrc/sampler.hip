@@ -64,6 +64,7 @@ __device__ __forceinline__ float block_max_1024(float v, float* red) {
 // index-order selection (top-p off), which needs a contiguous run of items per thread, goes through LDS.
 constexpr int kMaxRows = 64;      // 65535 elements / 1024 threads, rounded up; vocabularies up to 32768 take 32 (no spills)
 __host__ __device__ constexpr int staging_dwords_for(int n) { return ((n + 7) >> 3) * 4; }
+constexpr int kMaxVocab = 1 << 20;  // above 65535 entries the large-vocabulary kernels take over
 constexpr int kLdsVocab = 49152;  // the index-order selection holds vocabularies up to here in LDS (96 KB of fp16 values)
 
 __host__ __device__ inline int staging_dwords(int n) { return n <= kLdsVocab ? staging_dwords_for(n) : 0; }
@@ -279,10 +280,14 @@ __device__ __forceinline__ void select_in_index_order(const uint16_t* probs, int
 
 // sampler.h:94-107 + gpu_kernels.h:562-592, top-p: position in the descending stable order of the probabilities at
 // which the exact prefix sum, rounded to fp16, first reaches the threshold; the last position when none does.
-template <int NR>
-__device__ __forceinline__ void select_in_sorted_order(const Rows<NR>& x, int n, float threshold, unsigned int* hist32, const SampleOut out) {
-    // counts per probability value, two 16-bit counters per dword (n <= 65535)
-    auto hcount = [&](int b) -> unsigned int { return (hist32[b >> 1] >> (16 * (b & 1))) & 0xFFFFu; };
+// The items come from the thread's rows (vocabularies up to 65535: counters of 16 bits, two to a dword) or, WIDE, straight
+// from global memory with one 32-bit counter per value (larger vocabularies: plain loops, no staging).
+struct GlobalItems {
+    const uint16_t* bits;
+};
+template <bool WIDE, class Items>
+__device__ __forceinline__ void select_in_sorted_order(const Items& x, int n, float threshold, unsigned int* hist32, const SampleOut out) {
+    auto hcount = [&](int b) -> unsigned int { return WIDE ? hist32[b] : (hist32[b >> 1] >> (16 * (b & 1))) & 0xFFFFu; };
     __shared__ unsigned long long wave_totals[16];
     __shared__ unsigned int counts[kSampleThreads];
     __shared__ int s_best_thread;
@@ -299,23 +304,30 @@ __device__ __forceinline__ void select_in_sorted_order(const Rows<NR>& x, int n,
     }
     // histogram of the probability values.  Zeros (most of a peaked distribution) are counted per thread instead of
     // through the one LDS word they would all hit.
-    for (int b = tid; b < (kProbBins + 1) / 2; b += kSampleThreads) hist32[b] = 0u;
+    for (int b = tid; b < (WIDE ? kProbBins : (kProbBins + 1) / 2); b += kSampleThreads) hist32[b] = 0u;
     __syncthreads();
     unsigned int zeros = 0;
+    auto count_value = [&](uint32_t bits) {
+        const int b = min((int)bits, kProbBins - 1);
+        if (b == 0)
+            zeros++;
+        else if (WIDE)
+            atomicAdd(&hist32[b], 1u);
+        else
+            atomicAdd(&hist32[b >> 1], (b & 1) ? 0x10000u : 1u);
+    };
+    if constexpr (WIDE) {
+        for (int i = tid; i < n; i += kSampleThreads) count_value(x.bits[i]);
+    } else {
 #pragma unroll
-    for (int r = 0; r < NR; r++) {
-        if (r * kSampleThreads + tid < n) {
-            const int b = min((int)x.bits[r], kProbBins - 1);
-            if (b == 0)
-                zeros++;
-            else
-                atomicAdd(&hist32[b >> 1], (b & 1) ? 0x10000u : 1u);
+        for (int r = 0; r < (int)(sizeof(x.bits) / sizeof(x.bits[0])); r++) {
+            if (r * kSampleThreads + tid < n) count_value(x.bits[r]);
         }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) zeros += __shfl_xor(zeros, off);
     __syncthreads();
-    if (lane == 0 && zeros) atomicAdd(&hist32[0], zeros);  // bin 0 is the low half of word 0
+    if (lane == 0 && zeros) atomicAdd(&hist32[0], zeros);  // bin 0 is word 0, or its low half
     __syncthreads();
     // bins in descending order, a contiguous run per thread: thread 0 owns the largest values
     constexpr int BPT = (kProbBins + kSampleThreads - 1) / kSampleThreads;
@@ -392,31 +404,50 @@ __device__ __forceinline__ void select_in_sorted_order(const Rows<NR>& x, int n,
     }
     const int target_bin = s_bin;
     const unsigned int target_rank = s_rank;
-    // The target_rank-th element equal to target_bin, in index order (the radix sort is stable).  Index order is row by
-    // row, wave by wave, lane by lane: matches are counted per (row, wave) with a ballot, the counts scanned in that
-    // order, and the lane whose match has the wanted number reports its index.
-    counts[tid] = 0u;
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < NR; r++) {
-        if (r * kSampleThreads < n) {  // uniform
-            const bool m = r * kSampleThreads + tid < n && min((int)x.bits[r], kProbBins - 1) == target_bin;
-            const unsigned long long bal = __ballot(m);
-            if (lane == 0) counts[r * 16 + wave] = (unsigned int)__popcll(bal);
+    // The target_rank-th element equal to target_bin, in index order (the radix sort is stable).
+    if constexpr (WIDE) {
+        // a contiguous run of items per thread: matches counted per run, the counts scanned, and the thread whose run
+        // holds the wanted match walks it
+        const int per = (n + kSampleThreads - 1) / kSampleThreads;
+        const int i0 = min(tid * per, n), i1 = min(i0 + per, n);
+        unsigned int mine = 0;
+        for (int i = i0; i < i1; i++) mine += (min((int)x.bits[i], kProbBins - 1) == target_bin);
+        unsigned int seen = (unsigned int)block_exclusive_scan_1024((unsigned long long)mine, wave_totals);
+        if (seen < target_rank && seen + mine >= target_rank) {
+            for (int i = i0; i < i1; i++) {
+                if (min((int)x.bits[i], kProbBins - 1) == target_bin && ++seen == target_rank) {
+                    s_index = i;
+                    break;
+                }
+            }
         }
-    }
-    __syncthreads();
-    const unsigned int before_cell = (unsigned int)block_exclusive_scan_1024((unsigned long long)counts[tid], wave_totals);
-    counts[tid] = before_cell;  // (every thread rewrites the cell it read itself; the scan ended with a barrier)
-    __syncthreads();
+    } else {
+        // Index order is row by row, wave by wave, lane by lane: matches are counted per (row, wave) with a ballot, the
+        // counts scanned in that order, and the lane whose match has the wanted number reports its index.
+        constexpr int NR = (int)(sizeof(x.bits) / sizeof(x.bits[0]));
+        counts[tid] = 0u;
+        __syncthreads();
 #pragma unroll
-    for (int r = 0; r < NR; r++) {
-        if (r * kSampleThreads < n) {
-            const bool m = r * kSampleThreads + tid < n && min((int)x.bits[r], kProbBins - 1) == target_bin;
-            const unsigned long long bal = __ballot(m);
-            if (m) {
-                const unsigned int seen = counts[r * 16 + wave] + (unsigned int)__popcll(bal & ((1ull << lane) - 1ull));
-                if (seen + 1u == target_rank) s_index = r * kSampleThreads + tid;
+        for (int r = 0; r < NR; r++) {
+            if (r * kSampleThreads < n) {  // uniform
+                const bool m = r * kSampleThreads + tid < n && min((int)x.bits[r], kProbBins - 1) == target_bin;
+                const unsigned long long bal = __ballot(m);
+                if (lane == 0) counts[r * 16 + wave] = (unsigned int)__popcll(bal);
+            }
+        }
+        __syncthreads();
+        const unsigned int before_cell = (unsigned int)block_exclusive_scan_1024((unsigned long long)counts[tid], wave_totals);
+        counts[tid] = before_cell;  // (every thread rewrites the cell it read itself; the scan ended with a barrier)
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            if (r * kSampleThreads < n) {
+                const bool m = r * kSampleThreads + tid < n && min((int)x.bits[r], kProbBins - 1) == target_bin;
+                const unsigned long long bal = __ballot(m);
+                if (m) {
+                    const unsigned int seen = counts[r * 16 + wave] + (unsigned int)__popcll(bal & ((1ull << lane) - 1ull));
+                    if (seen + 1u == target_rank) s_index = r * kSampleThreads + tid;
+                }
             }
         }
     }
@@ -430,7 +461,34 @@ __global__ __launch_bounds__(kSampleThreads) void sample_sorted_kernel(const uin
     extern __shared__ unsigned int dyn_lds[];  // staging area, then the histogram
     Rows<NR> x;
     rows_load_staged(x, probs, n, reinterpret_cast<uint16_t*>(dyn_lds));
-    select_in_sorted_order(x, n, threshold, dyn_lds + staging_dwords(n), SampleOut{result, pPos, pPosGpu, mirror});
+    select_in_sorted_order<false>(x, n, threshold, dyn_lds + staging_dwords(n), SampleOut{result, pPos, pPosGpu, mirror});
+}
+
+// Vocabularies above 65535 entries (up to kMaxVocab): the same arithmetic in plain loops over global memory.
+__global__ __launch_bounds__(kSampleThreads) void softmax_logits_large_kernel(uint16_t* logits, int size, float temperature) {
+    __shared__ float red[16];
+    const int tid = threadIdx.x;
+    float max_val = -3.402823466e+38f;  // -FLT_MAX
+    for (int t = tid; t < size; t += kSampleThreads) {  // (a thread re-reads only what it wrote itself)
+        const uint16_t h = float_to_half_bits(half_bits_to_float(logits[t]) / temperature);
+        logits[t] = h;
+        max_val = fmaxf(max_val, half_bits_to_float(h));
+    }
+    max_val = block_max_1024(max_val, red);
+    float sum = 0.0f;
+    for (int t = tid; t < size; t += kSampleThreads) {
+        const float v = expf(half_bits_to_float(logits[t]) - max_val);
+        logits[t] = float_to_half_bits(v);
+        sum += v;
+    }
+    sum = block_sum_1024(sum, red);
+    for (int t = tid; t < size; t += kSampleThreads) logits[t] = float_to_half_bits(half_bits_to_float(logits[t]) / sum);
+}
+
+__global__ __launch_bounds__(kSampleThreads) void sample_sorted_large_kernel(const uint16_t* probs, int n, float threshold, int* result,
+                                                                             volatile int* pPos, int* pPosGpu, int* mirror) {
+    extern __shared__ unsigned int dyn_lds[];  // the histogram, one word per value
+    select_in_sorted_order<true>(GlobalItems{probs}, n, threshold, dyn_lds, SampleOut{result, pPos, pPosGpu, mirror});
 }
 
 __global__ __launch_bounds__(kSampleThreads) void sample_plain_kernel(const uint16_t* probs, int n, float threshold, int vec,
@@ -469,7 +527,7 @@ __global__ __launch_bounds__(kSampleThreads) void softmax_sample_kernel(uint16_t
     rows_softmax(x, n, temperature, red);
     rows_store_staged(logits, x, n, vals);
     if (SORTED) {
-        select_in_sorted_order(x, n, threshold, dyn_lds + staging_dwords(n), out);
+        select_in_sorted_order<false>(x, n, threshold, dyn_lds + staging_dwords(n), out);
     } else {
         // (launched for n <= kLdsVocab only: the staging area holds the probabilities)
         __syncthreads();
@@ -535,6 +593,10 @@ static int raise_sampler_lds(awq_ctx* ctx) {
 }
 
 static int launch_softmax_logits(awq_ctx* ctx, uint16_t* logits, int size, float temperature) {
+    if (size > 65535) {
+        hipLaunchKernelGGL(softmax_logits_large_kernel, dim3(1), dim3(kSampleThreads), 0, ctx->stream, logits, size, temperature);
+        return awq_check_launch("softmax_logits");
+    }
     if (int r = raise_sampler_lds(ctx)) return r;
     if (size <= 32 * kSampleThreads)
         hipLaunchKernelGGL(softmax_logits_kernel<32>, dim3(1), dim3(kSampleThreads), values_lds_bytes(size), ctx->stream, logits, size,
@@ -547,6 +609,11 @@ static int launch_softmax_logits(awq_ctx* ctx, uint16_t* logits, int size, float
 
 static int launch_sample(awq_ctx* ctx, const uint16_t* probs, int size, float threshold, int sorted, int* tokens,
                          volatile int* pos_host, int* pos_dev, int* mirror) {
+    if (sorted && size > 65535) {
+        hipLaunchKernelGGL(sample_sorted_large_kernel, dim3(1), dim3(kSampleThreads), (size_t)kProbBins * sizeof(unsigned int),
+                           ctx->stream, probs, size, threshold, tokens, pos_host, pos_dev, mirror);
+        return awq_check_launch("sample_top_p");
+    }
     if (int r = raise_sampler_lds(ctx)) return r;
     if (sorted) {
         const size_t lds = values_lds_bytes(size) + hist_lds_bytes();
@@ -593,7 +660,7 @@ int awq_sampler_run(awq_sampler* s, uint16_t* logits, int* tokens, volatile int*
         return awq_launch_argmax(s->ctx, logits, s->vocab_size, tokens, pos_host, pos_dev, gen_token, mirror);
     const bool nucleus = s->topp > 0.0f && s->topp < 1.0f;
     const float threshold = nucleus ? coin * s->topp : coin;
-    if (nucleus || s->vocab_size <= kLdsVocab)  // softmax and selection in one launch
+    if (nucleus ? s->vocab_size <= 65535 : s->vocab_size <= kLdsVocab)  // softmax and selection in one launch
         return launch_softmax_sample(s->ctx, logits, s->vocab_size, s->temperature, threshold, nucleus ? 1 : 0, tokens, pos_host,
                                      pos_dev, mirror);
     if (int r = launch_softmax_logits(s->ctx, logits, s->vocab_size, s->temperature)) return r;
@@ -613,7 +680,7 @@ int awq_sample_top_p(awq_ctx* ctx, const uint16_t* probs, int size, float thresh
                      volatile int* pos_host, int* pos_dev) {
     if (int r = awq_bind(ctx)) return r;
     AWQ_REQUIRE(probs && tokens && pos_host && pos_dev && size > 0, AWQ_ERR_ARG, "null pointer or empty vector");
-    AWQ_REQUIRE(size <= 65535, AWQ_ERR_SHAPE, "vocabularies above 65535 entries are not supported by the sampler");
+    AWQ_REQUIRE(size <= kMaxVocab, AWQ_ERR_SHAPE, "vocabularies above 1048576 entries are not supported by the sampler");
     return launch_sample(ctx, probs, size, threshold, sorted, tokens, pos_host, pos_dev, nullptr);
 }
 
@@ -621,7 +688,7 @@ int awq_sampler_create(awq_ctx* ctx, int vocab_size, float temperature, float to
                        awq_sampler** out) {
     if (int r = awq_bind(ctx)) return r;
     AWQ_REQUIRE(out && vocab_size > 0, AWQ_ERR_ARG, "null out or empty vocabulary");
-    AWQ_REQUIRE(vocab_size <= 65535, AWQ_ERR_SHAPE, "vocabularies above 65535 entries are not supported by the sampler");
+    AWQ_REQUIRE(vocab_size <= kMaxVocab, AWQ_ERR_SHAPE, "vocabularies above 1048576 entries are not supported by the sampler");
     AWQ_REQUIRE(temperature >= 0.0f, AWQ_ERR_ARG, "negative temperature");
     awq_sampler* s = new (std::nothrow) awq_sampler();
     AWQ_REQUIRE(s, AWQ_ERR_ARG, "out of host memory");

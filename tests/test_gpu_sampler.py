@@ -41,7 +41,7 @@ def _logits(seed, n, scale):
     return (np.random.default_rng(seed).normal(0, scale, n)).astype(np.float16)
 
 
-@pytest.mark.parametrize("n,temperature,scale", [(32000, 0.5, 2.0), (32000, 1.0, 5.0), (1000, 0.7, 1.0), (5, 0.3, 1.0), (1025, 2.0, 8.0), (65535, 0.9, 3.0), (40000, 0.7, 2.0), (32768, 0.6, 3.0), (32769, 0.6, 3.0)])
+@pytest.mark.parametrize("n,temperature,scale", [(32000, 0.5, 2.0), (32000, 1.0, 5.0), (1000, 0.7, 1.0), (5, 0.3, 1.0), (1025, 2.0, 8.0), (65535, 0.9, 3.0), (40000, 0.7, 2.0), (32768, 0.6, 3.0), (32769, 0.6, 3.0), (65536, 0.8, 3.0), (128256, 0.7, 4.0)])
 def test_softmax_logits(ctx, n, temperature, scale):
     l = _logits(3, n, scale)
     d = ctx.upload(l.view(np.uint16))
@@ -60,16 +60,16 @@ def _oracle_pick(probs, threshold, sorted_):
 
 
 @pytest.mark.parametrize("sorted_", [0, 1])
-@pytest.mark.parametrize("case", range(10))
+@pytest.mark.parametrize("case", range(12))
 def test_sample_top_p_identical_to_oracle(ctx, case, sorted_):
     rng = np.random.default_rng(200 + case)
-    n = [32000, 32000, 4097, 777, 64, 3, 65535, 1024, 40000, 49153][case]  # up to 32768 / 49152 / 65535: three forms of the kernels
+    n = [32000, 32000, 4097, 777, 64, 3, 65535, 1024, 40000, 49153, 65536, 128256][case]  # up to 32768 / 49152 / 65535 / beyond: the forms of the kernels
     if case == 7:
         probs = np.full(n, 1.0 / 1024, dtype=np.float16)  # all equal: pure tie-breaking by index
     elif case == 6:
         probs = oracle.softmax_logits(_logits(case, n, 0.2), 1.0)  # nearly flat: thousands of equal values per bin
     else:
-        probs = oracle.softmax_logits(_logits(case, n, [2.0, 7.0, 1.0, 3.0, 0.5, 1.0, 0, 0, 2.0, 4.0][case]), 0.8)
+        probs = oracle.softmax_logits(_logits(case, n, [2.0, 7.0, 1.0, 3.0, 0.5, 1.0, 0, 0, 2.0, 4.0, 0.3, 5.0][case]), 0.8)
     d = ctx.upload(probs.view(np.uint16))
     pin = Pinned(ctx)
     thresholds = list(rng.uniform(0, 1, 20)) + [0.0, 1e-8, 2.0 ** -24, 0.5, 0.999, 1.0, 1.0005, 1.5]
@@ -86,18 +86,19 @@ def test_sample_top_p_identical_to_oracle(ctx, case, sorted_):
 
 def test_sample_top_p_rejects_large_vocabulary(ctx):
     pin = Pinned(ctx)
-    d = ctx.zeros(70000 * 2)
+    d = ctx.zeros(16)
     with pytest.raises(A.AwqError) as e:
-        A.sample_top_p(ctx, d, 70000, 0.5, 1, pin.host + 16, pin.host, pin.dpos)
+        A.sample_top_p(ctx, d, (1 << 20) + 1, 0.5, 1, pin.host + 16, pin.host, pin.dpos)
     assert e.value.code == AWQ_ERR_SHAPE
     pin.close()
 
 
+@pytest.mark.parametrize("V", [32000, 128256])
 @pytest.mark.parametrize("temperature,topp", [(0.5, 0.6), (1.0, 0.9), (0.8, 1.0), (1.3, 0.0), (0.0, 0.6)])
-def test_sampler_object_follows_reference_sample(ctx, temperature, topp):
+def test_sampler_object_follows_reference_sample(ctx, temperature, topp, V):
     """awq_sampler_sample = coin from xorshift*, greedy when temperature is 0 or the token is not generated, else
     softmax + (top-p | plain) selection with threshold coin * topp | coin."""
-    V, seed = 32000, 4242
+    seed = 4242
     s = A.Sampler(ctx, V, temperature, topp, seed)
     state = np.array([seed], dtype=np.uint64)
     pin = Pinned(ctx)
