@@ -37,7 +37,8 @@ struct awq_ctx {
 constexpr int kAttnMaxHeads = 256;
 constexpr int kAttnFusedMaxSeq = 256;  // up to this launch size attention runs as one workgroup per head
 constexpr int kAttnMaxChunks = 4;      // ranges of positions whose partial P.V sums the O projection adds up
-constexpr int kAttnSplitMinSeq = 1024;  // launch sizes from which the fused schedule splits P.V over positions
+constexpr int kAttnSplitMinSeq = 1024;  // launch sizes from which the fused schedule splits P.V over positions ...
+constexpr int kAttnSplitMinRange = 320;  // ... if a range then covers at least this many positions of the launch size
 
 void awq_set_error(const char* fmt, ...);
 

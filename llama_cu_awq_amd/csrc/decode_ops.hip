@@ -599,6 +599,16 @@ int awq_launch_argmax(awq_ctx* ctx, const uint16_t* logits, int size, int* token
     return awq_check_launch("argmax");
 }
 
+// Internal: into how many ranges of positions the position-split P.V divides a head's rows: about one workgroup per
+// compute unit (heads x 64-dimension slices x ranges), each pulling whole cache lines.
+int awq_attention_partial_chunks(const awq_ctx* ctx, int num_heads, int head_size) {
+    const int slices = head_size >= 64 ? head_size / 64 : 1;
+    int chunks = ctx->cus / (num_heads * slices);
+    if (chunks < 1) chunks = 1;
+    if (chunks > kAttnMaxChunks) chunks = kAttnMaxChunks;
+    return chunks;
+}
+
 // Internal (fused schedule, launch sizes above kAttnFusedMaxSeq): scores, then P.V as fp32 partial sums over
 // `*chunks_out` ranges of positions, part[chunk][num_heads * head_size]; the consumer adds the chunks up in order and
 // rounds to fp16.  part must hold kAttnMaxChunks * num_heads * head_size floats.
@@ -608,10 +618,7 @@ int awq_launch_attention_partial(awq_ctx* ctx, float* part, int* chunks_out, con
     const int row_stride = num_heads * head_size / kv_mul;
     const float alpha = (float)(1.0 / sqrt((double)head_size));
     const int slices = head_size / 64;
-    // about one workgroup per compute unit, each pulling whole cache lines
-    int chunks = ctx->cus / (num_heads * slices);
-    if (chunks < 1) chunks = 1;
-    if (chunks > kAttnMaxChunks) chunks = kAttnMaxChunks;
+    const int chunks = awq_attention_partial_chunks(ctx, num_heads, head_size);
     const dim3 sgrid(div_up(max_seq_len, 64), num_heads);
     switch (head_size) {
         case 64: awq_launch(ctx, attn_scores_kernel<8>, sgrid, dim3(256), 0, att, q, key_cache, head_size, kv_mul, row_stride, alpha, pos); break;

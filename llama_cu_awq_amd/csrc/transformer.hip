@@ -23,6 +23,7 @@ int awq_launch_ffn(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const awq_qwe
                    int N, const uint16_t* norm_w, uint16_t* norm_out);
 int awq_launch_matvec_f16(awq_ctx* ctx, uint16_t* out, const uint16_t* x, const uint16_t* w, int n, int d,
                           const uint16_t* norm_w, uint16_t* norm_out);
+int awq_attention_partial_chunks(const awq_ctx* ctx, int num_heads, int head_size);
 int awq_launch_attention_partial(awq_ctx* ctx, float* part, int* chunks_out, const uint16_t* q, const uint16_t* key_cache,
                                  const uint16_t* value_cache, uint16_t* att, int num_heads, int head_size, int kv_mul,
                                  int max_seq_len, const int* pos);
@@ -526,7 +527,11 @@ int network_fused(awq_transformer* t, int seq_len_bin) {
         // reference's rounding point) while the O projection stages its input; xb is not written on this path.
         // (Measured: +1.4 % tokens/s at 1.6 K positions of the 13B shape; just above 256 positions the split costs
         // 2 us per layer more than it saves, so it starts at the 1024 bin.)
-        const bool split = seq_len_bin >= kAttnSplitMinSeq && dim <= 8192;
+        // ... and it needs ranges long enough to pay for the partial sums: with four ranges (32 heads) the 1024 bin is
+        // faster unsplit (7B shape at positions 600-664: 743 against 719 tokens/s), with three (40 heads) it is not
+        // (13B shape: 448 against 453); from the 2048 bin on the split wins at both
+        const bool split = seq_len_bin >= kAttnSplitMinSeq && dim <= 8192 &&
+                           seq_len_bin / awq_attention_partial_chunks(ctx, p.n_heads, head_size) >= kAttnSplitMinRange;
         int parts = 0;
         {
             LaunchProbe probe(t, LK_ATTENTION);
