@@ -608,6 +608,8 @@ int ensure_captured(awq_transformer* t, int mode, int graph_index, int seq_len_b
         awq_set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
         return AWQ_ERR_HIP;
     }
+    // (the first replay of an instantiated graph otherwise pays for its upload to the device, a few milliseconds)
+    (void)hipGraphUpload(*exec, ctx->stream);
     *done = true;
     return AWQ_OK;
 }
