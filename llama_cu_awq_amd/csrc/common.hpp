@@ -103,6 +103,9 @@ static inline int packed_zeros_height(int K) { return div_up(scales_height(K), 8
 // Largest reduction length the matrix-vector kernels stage in LDS (fp16
 // activations, 2 bytes each, inside the 64 KB a workgroup may allocate).
 constexpr int kMaxStagedK = 28672;
+// The int4 kernels take rows up to here (68 bytes of LDS per 32 elements: 136 KB of the compute unit's 160 KB; above
+// 64 KB a kernel's limit is raised on its first such launch on a device).
+constexpr int kMaxStagedKInt4 = 65536;
 
 // ---------------------------------------------------------------- device side
 #ifdef __HIPCC__

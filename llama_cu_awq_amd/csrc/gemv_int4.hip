@@ -17,6 +17,10 @@
 // scale (times 2^20) is applied once per 32 elements.
 #include <math.h>
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 #include "common.hpp"
 #include "gemv_core.hpp"
 
@@ -391,8 +395,8 @@ int check_shape(int K, int N) {
         awq_set_error("matrix of K=%d N=%d exceeds the 4 GiB that 32-bit row offsets address", K, N);
         return AWQ_ERR_SHAPE;
     }
-    if (K > kMaxStagedK) {
-        awq_set_error("K=%d exceeds the %d activations the kernels stage in LDS", K, kMaxStagedK);
+    if (K > kMaxStagedKInt4) {
+        awq_set_error("K=%d exceeds the %d activations the kernels stage in LDS", K, kMaxStagedKInt4);
         return AWQ_ERR_SHAPE;
     }
     return AWQ_OK;
@@ -435,6 +439,24 @@ int g_stamps_stride = 0, g_stamps_launches = 0, g_stamps_next = 0;
 int g_stamps_grid[4096], g_stamps_bytes[4096];
 #endif
 
+// Rows above 30 K elements need more dynamic LDS than a kernel may take by default (64 KB): the limit of the kernel
+// about to be launched is raised, once per device and kernel.
+std::mutex g_lds_mutex;
+std::set<std::pair<int, const void*>> g_lds_raised;
+int ensure_lds_limit(awq_ctx* ctx, const void* kernel, size_t lds, const char* what) {
+    if (lds <= 64 * 1024) return AWQ_OK;
+    std::lock_guard<std::mutex> lock(g_lds_mutex);
+    const auto key = std::make_pair(ctx->device, kernel);
+    if (g_lds_raised.count(key)) return AWQ_OK;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)(kMaxStagedKInt4 / 32) * 68));
+    if (e != hipSuccess) {
+        awq_set_error("%s: hipFuncSetAttribute(dynamic LDS) failed: %s", what, hipGetErrorString(e));
+        return AWQ_ERR_HIP;
+    }
+    g_lds_raised.insert(key);
+    return AWQ_OK;
+}
+
 template <int W, int R, int D, int KIND, bool ROPE, int SPLIT = 1>
 int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     const int groups_total = div_up(p.N, W * R * SPLIT);
@@ -473,6 +495,7 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
     const size_t lds = (size_t)p.C * 68;  // activations + per-chunk constant
     if constexpr (KIND == KIND_SINGLE && !ROPE && R == 1 && (W == 8 || W == 10 || W == 13)) {  // (partial-sum input comes with K <= 8192)
         if (p.xpart) {
+            if (int r = ensure_lds_limit(ctx, (const void*)gemv_int4_kernel<W, R, D, KIND, false, false, true, SPLIT>, lds, what)) return r;
             awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, false, true, SPLIT>, grid, dim3(W * 64), lds, p);
             return awq_check_launch(what);
         }
@@ -481,10 +504,13 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
         awq_set_error("%s: no kernel takes partial-sum input in this geometry", what);
         return AWQ_ERR_ARG;
     }
-    if (p.norm_w)
+    if (p.norm_w) {
+        if (int r = ensure_lds_limit(ctx, (const void*)gemv_int4_kernel<W, R, D, KIND, true, ROPE, false, SPLIT>, lds, what)) return r;
         awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, true, ROPE, false, SPLIT>, grid, dim3(W * 64), lds, p);
-    else
+    } else {
+        if (int r = ensure_lds_limit(ctx, (const void*)gemv_int4_kernel<W, R, D, KIND, false, ROPE, false, SPLIT>, lds, what)) return r;
         awq_launch(ctx, gemv_int4_kernel<W, R, D, KIND, false, ROPE, false, SPLIT>, grid, dim3(W * 64), lds, p);
+    }
     return awq_check_launch(what);
 }
 

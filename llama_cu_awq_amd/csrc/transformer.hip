@@ -148,7 +148,7 @@ int check_config(const awq_config& c) {
     // load correctly in the reference (weight_packer.cpp:156 vs llama2_q4.cu:111).
     AWQ_REQUIRE(c.dim % 32 == 0 && c.hidden_dim % 32 == 0, AWQ_ERR_SHAPE, "dim and hidden_dim must be multiples of 32");
     AWQ_REQUIRE((kv_dim & 7) == 0 && (c.vocab_size & 7) == 0, AWQ_ERR_SHAPE, "kv_dim and vocab_size must be multiples of 8");
-    AWQ_REQUIRE(c.dim <= kMaxStagedK && c.hidden_dim <= kMaxStagedK, AWQ_ERR_SHAPE, "dim/hidden_dim above the staged maximum");
+    AWQ_REQUIRE(c.dim <= kMaxStagedK && c.hidden_dim <= kMaxStagedKInt4, AWQ_ERR_SHAPE, "dim/hidden_dim above the staged maximum");
     const int head = c.dim / c.n_heads;
     AWQ_REQUIRE(head == 64 || head == 128 || head == 256, AWQ_ERR_SHAPE, "head size must be 64, 128 or 256");
     AWQ_REQUIRE(c.n_heads <= kAttnMaxHeads, AWQ_ERR_SHAPE, "too many heads");

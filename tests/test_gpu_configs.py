@@ -457,6 +457,30 @@ def test_70b_shape_grouped_queries_four_layers_matches_oracle(ctx):
         o.close()
 
 
+def test_405b_shape_grouped_queries_two_layers_matches_oracle(ctx):
+    """Llama-3.1-405B's layer shape (dim 16384, hidden 53248, 128 heads sharing 8 KV heads), two layers: rows of 53248
+    elements in the down projection take 113 KB of LDS per workgroup, beyond the 64 KB a kernel may use unless its limit
+    is raised; the first launches here are recorded ones."""
+    cfg = dict(dim=16384, hidden_dim=53248, n_layers=2, n_heads=128, n_kv_heads=8, vocab_size=4096, seq_len=128, rope_theta=500000.0)
+    img = synth.make_model_image(cfg, seed=405, threads=THREADS, scale_mult=0.25)
+    t = A.Transformer(ctx, image=img)
+    o = oracle.Model(img)
+    try:
+        n_prompt, steps = 4, 4 + 8
+        prompt = synth.prompt_tokens(405, n_prompt, cfg["vocab_size"])
+        o.reset(prompt)
+        ref = _oracle_record(o, n_prompt, steps)
+        assert all(np.isfinite(l.astype(np.float32)).all() for l, _ in ref)
+        for mode, graph in ((A.SCHEDULE_FUSED, True), (A.SCHEDULE_FUSED, False), (A.SCHEDULE_REFERENCE, False)):
+            t.reset(prompt)
+            _, errs, ties = _gpu_record(t, n_prompt, steps, graph, mode, ref=ref)
+            assert max(errs) <= 1e-2, (mode, graph, max(errs))
+            assert ties <= 3, ties
+    finally:
+        t.close()
+        o.close()
+
+
 def test_33b_full_model_schedules_agree_and_stay_finite(ctx):
     """All 60 layers (17.5 GB of weights on the one GPU): the oracle would need minutes, so the check is that the two
     multi-kernel schedules, which share no matrix-vector launch geometry for the norm-fused steps, produce the same

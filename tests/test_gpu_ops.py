@@ -68,7 +68,7 @@ def test_matvec_int4_plain(ctx, K, N):
 # four rows side by side in a wave, two or three passes in flight, partly filled last workgroups and row groups, row
 # lengths that are no multiple of a pass or of a quantisation group), in the three forms.
 SWEEP_K = [8, 96, 136, 256, 512, 544, 1000, 2560, 2592, 3072, 4096, 5120, 6144, 6656, 8192, 8224, 10240, 11008, 13824, 17920, 20480,
-           28672]
+           28672, 28704, 53248, 65536]  # the last three: more than 64 KB of LDS per workgroup
 SWEEP_N = [8, 40, 264, 1000]
 
 
@@ -357,7 +357,7 @@ def test_ffn_matvec_silu(ctx, K, N):
     assert_close_f16(got, f16(want), ulps=4)
 
 
-@pytest.mark.parametrize("K,N", [(12, 8), (8, 12), (4096, 4100), (0, 8)])
+@pytest.mark.parametrize("K,N", [(12, 8), (8, 12), (4096, 4100), (0, 8), (65568, 8)])
 def test_shape_guard(ctx, K, N):
     """The reference prints 'Unsupported matmul size' and exits; the library returns AWQ_ERR_SHAPE."""
     buf = ctx.alloc(1 << 16)
