@@ -468,6 +468,10 @@ int launch(awq_ctx* ctx, GemvParams& p, int grid_y, const char* what) {
         const int cus = ctx->cus;
         if (gx > 3 * cus) gx = 3 * cus;
     }
+    // Rows so long that their staged activations leave room for one workgroup per compute unit (more than 64 KB of LDS):
+    // one workgroup per compute unit walks the row groups and stages the activations once, instead of once per group
+    // (K = 53248, N = 16384: 100 -> 93 us).
+    if ((size_t)p.C * 68 > 64 * 1024 && grid_y == 1 && gx > ctx->cus) gx = ctx->cus;
     p.gx = gx;
     p.groups_q = groups_total / gx;
     p.groups_rem = groups_total % gx;

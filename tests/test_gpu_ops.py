@@ -17,7 +17,8 @@ from tests.helpers import assert_close_f16, f16, rel_l2, ulp_diff_f16
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (5120, 5120), (13824, 5120), (6656, 1024), (17920, 512), (128, 8), (200, 24), (1056, 40)]
+SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (5120, 5120), (13824, 5120), (6656, 1024), (17920, 512), (128, 8), (200, 24), (1056, 40),
+          (53248, 4608)]  # the last: rows so long that one workgroup per compute unit walks the row groups (288 groups on 256 units)
 
 
 def _case(K, N, tag=0):
