@@ -5,6 +5,7 @@ dequantised weights (the stated bound) and, tighter, within 2 fp16 steps of the 
 (summation order differs); fp16 element-wise ops within 1 fp16 step of the oracle.
 """
 import ctypes as C
+import functools
 
 import numpy as np
 import pytest
@@ -21,11 +22,23 @@ SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096), (5120, 5120), (13824, 5120
           (53248, 4608)]  # the last: rows so long that one workgroup per compute unit walks the row groups (288 groups on 256 units)
 
 
+@functools.lru_cache(maxsize=16)
 def _case(K, N, tag=0):
     key = synth.stream_key(0, "case", K, N, tag)
     w, z, s = synth.make_qweight(key, K, N)
     x = synth.normal_f16(synth.stream_key(key, "x"), K)
+    for a in (w, z, s, x):
+        a.setflags(write=False)  # shared between the tests that ask for the same case
     return w, z, s, x
+
+
+@functools.lru_cache(maxsize=6)
+def _exact(K, N, tag):
+    """The exactly dequantised matrix of _case(K, N, tag) in fp64 (kept across the parametrisations that reuse it)."""
+    w, z, s, _ = _case(K, N, tag)
+    m = synth.dequantize(w, z, s, K)
+    m.setflags(write=False)
+    return m
 
 
 @pytest.mark.parametrize("K,N", [(4096, 512), (11008, 64), (200, 24), (128, 8), (13824, 32)])
@@ -141,7 +154,7 @@ def test_matvec_int4_scaled_activations(ctx, K, N, e):
     dout = ctx.zeros(N * 2)
     A.matmul_q(ctx, dout, ctx.upload(x), qw, K, N)
     got = f16(dout.download(np.uint16))
-    truth = synth.dequantize(w, z, s, K) @ x.astype(np.float64)
+    truth = _exact(K, N, 30) @ x.astype(np.float64)
     floor = _fp16_rounding_floor(truth)
     assert floor <= 5e-4  # the outputs are representable: the stated bound applies as it is
     assert rel_l2(got, truth) <= 1e-3
@@ -174,8 +187,8 @@ def test_qkv_matvec_scaled_activations(ctx, K, N, e):
     oracle.qkv_matvec(q, kc, vc, x, *mats, K, N, loff, pos)
     for got, want in ((dq.download(np.uint16), q), (dk.download(np.uint16), kc), (dv.download(np.uint16), vc)):
         assert_close_f16(f16(got), f16(want), ulps=2)
-    for got, m in ((dq.download(np.uint16), mats[0]), (dv.download(np.uint16)[pos * N : (pos + 1) * N], mats[2])):
-        truth = synth.dequantize(*m, K) @ x.astype(np.float64)
+    for got, tag in ((dq.download(np.uint16), 31), (dv.download(np.uint16)[pos * N : (pos + 1) * N], 33)):
+        truth = _exact(K, N, tag) @ x.astype(np.float64)
         assert rel_l2(f16(got), truth) <= 1e-3
 
 
@@ -197,8 +210,8 @@ def test_ffn_matvec_silu_scaled_activations(ctx, K, N, e):
     assert np.isfinite(f16(want).astype(np.float32)).all()
     assert_close_f16(got, f16(want), ulps=4)
     xd = x.astype(np.float64)
-    g = synth.dequantize(*gate, K) @ xd
-    u = synth.dequantize(*up, K) @ xd
+    g = _exact(K, N, 35) @ xd
+    u = _exact(K, N, 36) @ xd
     truth = g / (1.0 + np.exp(-g)) * u
     assert rel_l2(got, truth) <= 1e-3 + _fp16_rounding_floor(truth)
 
