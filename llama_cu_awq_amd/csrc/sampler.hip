@@ -405,7 +405,21 @@ __device__ __forceinline__ void select_in_sorted_order(const Items& x, int n, fl
     const int target_bin = s_bin;
     const unsigned int target_rank = s_rank;
     // The target_rank-th element equal to target_bin, in index order (the radix sort is stable).
-    if constexpr (WIDE) {
+    bool unique = false;
+    if constexpr (!WIDE) {
+        // the usual case when the crossing lies among the likely tokens: the value occurs once, and whoever holds it
+        // reports its index (no counting, no scan)
+        unique = hcount(target_bin) == 1u;
+        if (unique) {
+            constexpr int NR = (int)(sizeof(x.bits) / sizeof(x.bits[0]));
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                if (r * kSampleThreads + tid < n && min((int)x.bits[r], kProbBins - 1) == target_bin) s_index = r * kSampleThreads + tid;
+            }
+        }
+    }
+    if (unique) {
+    } else if constexpr (WIDE) {
         // a contiguous run of items per thread: matches counted per run, the counts scanned, and the thread whose run
         // holds the wanted match walks it
         const int per = (n + kSampleThreads - 1) / kSampleThreads;
