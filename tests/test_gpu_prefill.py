@@ -114,15 +114,21 @@ def test_prefill_in_two_parts_equals_one(ctx):
 CFG_LONG2K = dict(dim=256, hidden_dim=512, n_layers=2, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=2176, rope_theta=10000.0)
 
 
-def test_prefill_past_the_batched_attention_bound(ctx):
-    cfg, n_prompt = CFG_LONG2K, 2000
+# the same with grouped queries: four heads share one KV head (the position-split attention and the single QKV launch
+# with fewer K and V rows, at long context)
+CFG_LONG2K_GQA = dict(dim=512, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=1, vocab_size=512, seq_len=2176, rope_theta=10000.0)
+
+
+@pytest.mark.parametrize("cfg", [CFG_LONG2K, CFG_LONG2K_GQA], ids=["2-heads", "grouped-queries"])
+def test_prefill_past_the_batched_attention_bound(ctx, cfg):
+    n_prompt = 2000
     img = synth.make_model_image(cfg, seed=33, scale_mult=0.5)
     prompt = synth.prompt_tokens(33, n_prompt, cfg["vocab_size"])
     o = oracle.Model(img)
     o.reset(prompt)
     for i in range(n_prompt):
         o.forward(i >= n_prompt - 1)
-    kv_dim, L, seq, vocab = cfg["dim"], cfg["n_layers"], cfg["seq_len"], cfg["vocab_size"]
+    kv_dim, L, seq, vocab = cfg["dim"] * cfg["n_kv_heads"] // cfg["n_heads"], cfg["n_layers"], cfg["seq_len"], cfg["vocab_size"]
     want_kv = {n: f16(o.buffer(n, L * seq * kv_dim)).reshape(L, seq, kv_dim)[:, :n_prompt].copy() for n in ("key_cache", "value_cache")}
     want_logits = f16(o.buffer("logits", vocab)).copy()
     want_next = o.tokens(n_prompt + 1)[n_prompt]
