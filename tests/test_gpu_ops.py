@@ -280,7 +280,7 @@ def test_matvec_int4_accum_and_kv_offset(ctx, K, N):
 
 def test_zero_weights_leave_residual(ctx):
     """accum with W == 0 (q == z everywhere) returns the residual.  The kernel forms sum q*x - z * sum x with each sum
-    rounded in fp32 on its own, so W x comes out as fp32 rounding noise (around 1e-7 here) instead of an exact zero:
+    rounded in fp32 on its own, so W x comes out as fp32 rounding noise (about 1e-7 here) instead of an exact zero:
     the residual comes back bit for bit except where that noise crosses an fp16 rounding boundary (one step)."""
     K, N = 256, 64
     pwh, pzh, sh = synth.strides(K)
